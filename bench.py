@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the optimizer-step hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4] [--no-cpu-baseline]
+
+A "step" is one fused AdamW update over one synthetic partition that is already resident in HBM.
+Default workload: the Llama-7B decoder-layer partition (202,383,360 elements, bf16 gradients,
+AdamW at t=100, bf16 copy-out). Prints ONE JSON line: whole-job elements/s, the roofline of the
+update kernel (algorithmic bytes / measured kernel time against 8 TB/s) and the reference CPU
+Adam timed on this machine's host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+N_7B_LAYER = 4 * 4096 ** 2 + 3 * 4096 * 11008 + 2 * 4096                    # 202,383,360
+N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 855,654,400
+
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
+# profiles/); None until measured for a workload.
+MEASURED_TRAFFIC_BYTES = {"cfg2": None, "cfg3": None, "cfg4": None}
+
+HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
+
+
+def percentile_mean(samples, lo=0.2, hi=0.8):
+    """Mean of the 20th..80th percentile band, the reference's own statistic
+    (flextrain/auto_config.py:48-55)."""
+    s = sorted(samples)
+    a, b = int(len(s) * lo), max(int(len(s) * hi), int(len(s) * lo) + 1)
+    band = s[a:b]
+    return sum(band) / len(band)
+
+
+def make_inputs(torch, n, g_dtype, g_std, device, scale=1.0):
+    gen = torch.Generator(device=device).manual_seed(0)
+    p = torch.randn(n, device=device, generator=gen) * 0.02
+    m = torch.randn(n, device=device, generator=gen) * 1e-4
+    v = torch.rand(n, device=device, generator=gen) * 1e-6
+    g = (torch.randn(n, device=device, generator=gen) * (g_std * scale)).to(g_dtype)
+    h = torch.empty(n, dtype=torch.bfloat16, device=device)
+    return p, g, m, v, h
+
+
+def cpu_baseline(n, budget_s=20.0):
+    """Times the reference CPU Adam (its own C++ compiled into oracle/_ref when present, else this
+    repository's restatement) on host buffers of the workload's size: fp32 gradients and an fp16
+    copy-out, the only form the reference supports. 1 warm-up call, then timed calls until the
+    budget is used (at least 3, at most 20); 20-80 percentile mean, as flextrain/auto_config.py
+    does for its own optimizer probe."""
+    import numpy as np
+    import torch
+
+    import oracle
+    threads = oracle.max_threads()
+    ref = oracle.reference_module()
+    tp = torch.randn(n) * 0.02
+    tg = torch.randn(n) * 1e-3
+    tm = torch.zeros(n)
+    tv = torch.zeros(n)
+    th = torch.zeros(n, dtype=torch.float16)
+    if ref is not None:
+        kind, oid = "reference", 4242
+        ref.create_adam(oid, HP["lr"], *HP["betas"], HP["eps"], HP["weight_decay"], True, False)
+
+        def call(t):
+            ref.adam_update_copy(oid, t, HP["lr"], *HP["betas"], HP["eps"], HP["weight_decay"], True, tp, tg, tm, tv, th)
+    else:
+        kind = "port"
+        pn, gn, mn, vn = tp.numpy(), tg.numpy(), tm.numpy(), tv.numpy()
+        hn = th.numpy().view(np.uint16)
+
+        def call(t):
+            oracle.adam_step(pn, gn, mn, vn, step=t, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
+                             weight_decay=HP["weight_decay"], half_out=hn, half_dtype=oracle.F16)
+    call(1)
+    times, t_begin = [], time.perf_counter()
+    while len(times) < 20 and (len(times) < 3 or time.perf_counter() - t_begin < budget_s):
+        t0 = time.perf_counter()
+        call(len(times) + 2)
+        times.append(time.perf_counter() - t0)
+    if ref is not None:
+        ref.destroy_adam(oid)
+    sec = percentile_mean(times)
+    return {
+        "value": n / sec, "unit": "elements/s", "cores": threads, "kind": kind,
+        "sample": f"{len(times)} timed calls (1 warm-up) of the CPU Adam with fp16 copy-out on {n} fp32 elements "
+                  f"in host memory, {threads} OpenMP threads, 20-80 percentile mean",
+        "ms_per_call": sec * 1e3, "host_gbps": n * 30 / sec / 1e9,
+        "flavour": getattr(ref, "flavour", f"libftoracle isa={oracle.best_isa()}"),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures the optimizer step of ONE GPU's partition; --gpus must be 1 "
+              "(the path shards by giving each GPU its own slice; no multi-GPU figure exists).", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 1
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.loss_scaler import GradientGuard
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    eng = FlexTrainCPUAdam(**HP)
+
+    if args.workload == "cfg2":
+        n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.bfloat16, 100, 1.0, None
+        p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev)
+        name = "cfg2: Llama-7B decoder-layer partition resident in HBM, bf16 grads, AdamW t=100, bf16 copy-out"
+        bytes_per_elem, stats_pass = 28, False
+    elif args.workload == "cfg3":
+        n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.float16, 100, 65536.0, None
+        p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev, scale=scale)
+        name = "cfg3: 7B-layer partition, fp16 grads x65536, fused overflow check + unscale + AdamW (no overflow)"
+        bytes_per_elem, stats_pass = 28, True
+    else:
+        n, g_dtype, t_step, scale, max_norm = N_70B_LAYER, torch.bfloat16, 1000, 1.0, 1.0
+        p, g, m, v, h = make_inputs(torch, n, g_dtype, 5e-3, dev)
+        name = "cfg4: Llama-70B-shaped layer partition, bf16 grads, global-norm clip to 1.0 + AdamW t=1000"
+        bytes_per_elem, stats_pass = 28, True
+
+    guard = GradientGuard(dev) if stats_pass else None
+    group = {"step": t_step}
+
+    def one_step():
+        if guard is not None:
+            guard.begin()
+            guard.add(g, loss_scale=scale)
+            ctl = guard.decide_async(loss_scale=scale, max_grad_norm=max_norm)
+            eng._step(group, h, p, g, m, v, control=ctl)
+        else:
+            eng._step(group, h, p, g, m, v)
+
+    for _ in range(args.warmup):
+        one_step()
+    torch.cuda.synchronize()
+
+    # Per-launch HIP events on the stream the kernels run on (torch's current stream), recorded
+    # inside the timed region: ev[i][0] before the update kernel, ev[i][1] after it.
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        ev[i][0].record()
+        if guard is not None:
+            guard.begin()
+            guard.add(g, loss_scale=scale)
+            ctl = guard.decide_async(loss_scale=scale, max_grad_norm=max_norm)
+            ev[i][1].record()
+            eng._step(group, h, p, g, m, v, control=ctl)
+        else:
+            ev[i][1].record()
+            eng._step(group, h, p, g, m, v)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    upd_ms = [e[1].elapsed_time(e[2]) for e in ev]
+    pre_ms = [e[0].elapsed_time(e[1]) for e in ev]
+    upd_avg = sum(upd_ms) / len(upd_ms)
+    ms_per_step = wall * 1e3 / args.steps
+    alg_bytes = n * bytes_per_elem
+    achieved = alg_bytes / (upd_avg * 1e-3) / 1e9
+    out = {
+        "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
+        "value": n / (ms_per_step * 1e-3),
+        "unit": "elements/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": name, "elements": n, "grad_dtype": str(g_dtype).replace("torch.", ""),
+                   "copy_dtype": "bfloat16", "bytes_per_element": bytes_per_elem},
+        "hbm_gbps": achieved,
+        "hbm_frac_of_peak": achieved / HBM_PEAK_GBPS,
+        "roofline": {
+            "bound": "hbm", "kernel": "adam_vec_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES[args.workload],
+            "algorithmic_bytes_per_launch": alg_bytes, "kernel_ms_avg": upd_avg, "kernel_ms_min": min(upd_ms),
+            "kernel_ms_p20_80": percentile_mean(upd_ms),
+        },
+    }
+    if stats_pass:
+        pre_avg = sum(pre_ms) / len(pre_ms)
+        out["stats_pass"] = {"kernel": "grad_stats_kernel", "ms_avg": pre_avg, "bytes": n * 2,
+                             "achieved_gbps": n * 2 / (pre_avg * 1e-3) / 1e9}
+    if not args.no_cpu_baseline:
+        del p, g, m, v, h
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline(n)
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

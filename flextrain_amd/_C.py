@@ -1,0 +1,93 @@
+"""ctypes binding of libftadam.so -- the only way Python reaches the HIP kernels.
+
+There is no Python or CPU fallback: if the library has not been built, or a call fails, an
+exception is raised. Signatures mirror ``include/ft_adam.h`` one to one.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_uint64, c_void_p
+
+import torch
+
+F32, F16, BF16 = 0, 1, 2
+
+DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libftadam.so")
+
+EXPORTS = {
+    # name: (restype, argtypes)
+    "ft_last_error": (c_char_p, []),
+    "ft_abi_version": (c_int, []),
+    "ft_device_count": (c_int, []),
+    "ft_adam_create": (c_int, [c_int, c_float, c_float, c_float, c_float, c_float, c_int, c_int]),
+    "ft_adam_destroy": (c_int, [c_int]),
+    "ft_adam_step": (c_int, [c_int, c_uint64, c_float, c_float, c_float, c_float, c_float, c_int, c_float,
+                             c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_size_t,
+                             c_void_p, c_void_p]),
+    "ft_grad_stats_workspace_bytes": (c_size_t, []),
+    "ft_grad_stats": (c_int, [c_void_p, c_int, c_size_t, c_float, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "ft_grad_control": (c_int, [c_void_p, c_float, c_float, c_void_p, c_void_p]),
+    "ft_pinned_alloc": (c_int, [c_size_t, POINTER(c_void_p)]),
+    "ft_pinned_free": (c_int, [c_void_p]),
+    "ft_offload_create": (c_int, [c_size_t, c_int, POINTER(c_void_p)]),
+    "ft_offload_destroy": (c_int, [c_void_p]),
+    "ft_offload_step": (c_int, [c_void_p, c_int, c_uint64, c_float, c_float, c_float, c_float, c_float, c_int,
+                                c_float, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                c_int, c_size_t, c_void_p, c_void_p]),
+    "ft_offload_wait": (c_int, [c_void_p]),
+    "ft_offload_elapsed_ms": (c_int, [c_void_p, POINTER(c_float)]),
+    "ft_link_bandwidth": (c_int, [c_size_t, c_int, c_int, POINTER(c_double)]),
+    "ft_set_launch_tuning": (c_int, [c_int, c_int]),
+}
+
+
+class FtError(RuntimeError):
+    """A libftadam.so entry point returned a negative code."""
+
+    def __init__(self, fn: str, code: int, message: str):
+        super().__init__(f"{fn} failed ({code}): {message}")
+        self.code = code
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Loads the library on first use. Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m flextrain_amd.build` "
+                "(hipcc, gfx950). There is no CPU fallback for the optimizer step.")
+        L = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def check(fn: str, rc: int) -> int:
+    if rc < 0:
+        msg = lib().ft_last_error()
+        err = FtError(fn, rc, msg.decode() if msg else "")
+        if rc in (-1, -2):  # FT_EINVAL, FT_EALIGN
+            raise ValueError(str(err))
+        raise err
+    return rc
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype}; expected float32, float16 or bfloat16") from None
+
+
+def current_stream_ptr(device=None) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

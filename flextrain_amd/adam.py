@@ -1,0 +1,221 @@
+"""Adam / AdamW on the GPU behind the reference's ``flextrain.ops.adam`` surface.
+
+``FlexTrainCPUAdam`` mirrors the reference class of that name (``flextrain/ops/adam/cpu_adam.py:17-135``):
+same constructor arguments and defaults, same ``_init_optimizer_states`` / ``_step`` contract, an
+optimizer id registered with the native library on construction and released on deletion.
+The native side is libftadam.so (hand-written gfx950 kernels) instead of the AVX/OpenMP extension,
+so the tensors handed to ``_step`` are GPU tensors (resident mode) or pinned host tensors that are
+streamed through the GPU in chunks (offloaded mode).
+
+``FlexTrainAdam`` mirrors ``flextrain/ops/adam/__init__.py:10-34``.
+
+Additions over the reference, all optional and neutral by default:
+  * gradients may be fp32, fp16 or bf16; the low-precision copy is written in *its own* dtype
+    (the reference writes fp16 bit patterns whatever the tensor's dtype, ``simd.h:35-37``);
+  * ``grad_mult`` (one fp32 multiply applied to each gradient element on load: unscale x clip) and
+    ``control`` (a device-side skip / multiplier decision) for mixed-precision training.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from typing import Dict, List, Optional
+
+import torch
+from torch import Tensor
+
+from . import _C
+from .optimizer import STEP_KEY, FlexTrainCPUOptimizer, FlexTrainOptimizer
+
+#: elements per chunk of the offloaded step (64 Mi elements = 256 MiB per fp32 array)
+DEFAULT_OFFLOAD_CHUNK = 64 * 1024 * 1024
+DEFAULT_OFFLOAD_SLOTS = 3
+
+
+def _flat(name: str, t: Tensor, dtype_ok, numel: int) -> Tensor:
+    if t.dtype not in dtype_ok:
+        raise ValueError(f"{name} has dtype {t.dtype}, expected one of {sorted(map(str, dtype_ok))}")
+    if t.numel() != numel:
+        raise ValueError(f"{name} has {t.numel()} elements, expected {numel}")
+    if not t.is_contiguous():
+        # The reference calls .contiguous() and then updates the temporary, losing the result
+        # (cpu_adam_impl.cpp:225-228); refusing is the only safe reading of "in place".
+        raise ValueError(f"{name} must be contiguous: the update is in place")
+    return t
+
+
+class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
+    """Fused Adam/AdamW step engine (GPU kernels; the class keeps its reference name)."""
+
+    optimizer_id = 0
+    _id_lock = threading.Lock()
+
+    def __init__(
+        self,
+        lr=1e-3,
+        bias_correction=True,
+        betas=(0.9, 0.999),
+        eps=1e-8,
+        weight_decay=0.01,
+        amsgrad=False,
+        adamw_mode=True,
+        *args,
+        offload_chunk_elems: int = DEFAULT_OFFLOAD_CHUNK,
+        offload_slots: int = DEFAULT_OFFLOAD_SLOTS,
+        should_log: bool = False,
+        **kwargs,
+    ):
+        # amsgrad is accepted and ignored, as in the reference (cpu_adam.py:63-66).
+        self.default_args = dict(
+            lr=lr, betas=betas, eps=eps, weight_decay=weight_decay,
+            bias_correction=bias_correction, amsgrad=amsgrad,
+        )
+        FlexTrainCPUOptimizer.__init__(self)
+        with FlexTrainCPUAdam._id_lock:
+            self.opt_id = FlexTrainCPUAdam.optimizer_id
+            FlexTrainCPUAdam.optimizer_id += 1
+        self.adam_w_mode = adamw_mode
+        self._lib = _C.lib()  # raises if the native library is missing: there is no fallback
+        self._offload_chunk = int(offload_chunk_elems)
+        self._offload_slots = int(offload_slots)
+        self._engine: Optional[ctypes.c_void_p] = None
+        _C.check("ft_adam_create", self._lib.ft_adam_create(
+            self.opt_id, lr, betas[0], betas[1], eps, weight_decay, int(bool(adamw_mode)), int(bool(should_log))))
+
+    def __del__(self):
+        try:
+            if self._engine is not None:
+                self._lib.ft_offload_destroy(self._engine)
+                self._engine = None
+            self._lib.ft_adam_destroy(self.opt_id)
+        except BaseException:
+            pass
+
+    def _set_defaults_args(self, group_args: Dict):
+        for k, v in self.default_args.items():
+            group_args.setdefault(k, v)
+
+    def _init_optimizer_states(self, numel: int, dtype: torch.dtype) -> List[Tensor]:
+        """exp_avg and exp_avg_sq, zero-filled, where the master state lives
+        (reference ``cpu_adam.py:104-106`` returns two pinned host tensors)."""
+        return [self._allocate(numel, dtype, "zeros") for _ in range(2)]
+
+    # ------------------------------------------------------------------------------------------
+    def _offload_engine(self) -> ctypes.c_void_p:
+        if self._engine is None:
+            handle = ctypes.c_void_p()
+            _C.check("ft_offload_create", self._lib.ft_offload_create(
+                self._offload_chunk, self._offload_slots, ctypes.byref(handle)))
+            self._engine = handle
+        return self._engine
+
+    def _step(
+        self, group_args: Dict,
+        half_parameter: Optional[Tensor], full_parameter: Tensor,
+        gradient: Tensor, *optimizer_states: Tensor,
+        grad_mult: float = 1.0,
+        control: Optional[Tensor] = None,
+        blocking: Optional[bool] = None,
+    ):
+        """One Adam/AdamW update of a contiguous segment, in place.
+
+        Same contract as the reference ``_step`` (``cpu_adam.py:108-135``): ``group_args`` must hold
+        ``"step"``; missing hyper-parameters are filled from the constructor's. With
+        ``half_parameter`` the new parameters are also written there in its dtype.
+
+        Resident mode (``full_parameter`` on the GPU): the kernel is enqueued on torch's current
+        stream and the call returns at once. Offloaded mode (``full_parameter`` in pinned host
+        memory): the chunk pipeline is enqueued; with ``blocking`` (default in this mode) the call
+        returns when the host arrays hold the new values, as the reference's host step does.
+        """
+        assert STEP_KEY in group_args, f"Key '{STEP_KEY}' not found in parameter group arguments."
+        self._set_defaults_args(group_args)
+        if len(optimizer_states) != 2:
+            raise ValueError("Adam needs exactly two optimizer states (exp_avg, exp_avg_sq)")
+        exp_avg, exp_avg_sq = optimizer_states
+        n = full_parameter.numel()
+        f32 = {torch.float32}
+        _flat("full_parameter", full_parameter, f32, n)
+        _flat("exp_avg", exp_avg, f32, n)
+        _flat("exp_avg_sq", exp_avg_sq, f32, n)
+        _flat("gradient", gradient, set(_C.DTYPE_CODE), n)
+        if half_parameter is not None:
+            _flat("half_parameter", half_parameter, {torch.float16, torch.bfloat16}, n)
+        if n == 0:
+            return
+        g_code = _C.dtype_code(gradient.dtype)
+        h_code = _C.dtype_code(half_parameter.dtype) if half_parameter is not None else _C.F16
+        h_ptr = half_parameter.data_ptr() if half_parameter is not None else None
+        ctl_ptr = None
+        if control is not None:
+            if not control.is_cuda or control.numel() * control.element_size() < 16:
+                raise ValueError("control must be a 16-byte device buffer (ft_step_control_t)")
+            ctl_ptr = control.data_ptr()
+        beta1, beta2 = group_args["betas"]
+        hyper = (int(group_args[STEP_KEY]), float(group_args["lr"]), float(beta1), float(beta2),
+                 float(group_args["eps"]), float(group_args["weight_decay"]),
+                 int(bool(group_args["bias_correction"])), float(grad_mult))
+
+        if full_parameter.is_cuda:
+            for name, t in (("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq), ("gradient", gradient),
+                            ("half_parameter", half_parameter)):
+                if t is not None and t.device != full_parameter.device:
+                    raise ValueError(f"{name} is on {t.device} but full_parameter is on {full_parameter.device}")
+            with torch.cuda.device(full_parameter.device):
+                _C.check("ft_adam_step", self._lib.ft_adam_step(
+                    self.opt_id, *hyper, full_parameter.data_ptr(), gradient.data_ptr(), g_code,
+                    exp_avg.data_ptr(), exp_avg_sq.data_ptr(), h_ptr, h_code, n, ctl_ptr,
+                    _C.current_stream_ptr(full_parameter.device)))
+            return
+
+        # offloaded: master state in pinned host memory
+        for name, t in (("full_parameter", full_parameter), ("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
+            if t.is_cuda or not t.is_pinned():
+                raise ValueError(f"{name} must be pinned host memory when full_parameter is on the host")
+        for name, t in (("gradient", gradient), ("half_parameter", half_parameter)):
+            if t is not None and not t.is_cuda and not t.is_pinned():
+                raise ValueError(f"{name} must be on the GPU or in pinned host memory")
+        g_on_host = int(not gradient.is_cuda)
+        h_on_host = int(half_parameter is not None and not half_parameter.is_cuda)
+        engine = self._offload_engine()
+        _C.check("ft_offload_step", self._lib.ft_offload_step(
+            engine, self.opt_id, *hyper, full_parameter.data_ptr(), gradient.data_ptr(), g_code, g_on_host,
+            exp_avg.data_ptr(), exp_avg_sq.data_ptr(), h_ptr, h_code, h_on_host, n, ctl_ptr,
+            _C.current_stream_ptr()))
+        if blocking is None or blocking:
+            _C.check("ft_offload_wait", self._lib.ft_offload_wait(engine))
+
+    def synchronize(self):
+        """Waits for the last offloaded step (no-op if none was enqueued)."""
+        if self._engine is not None:
+            _C.check("ft_offload_wait", self._lib.ft_offload_wait(self._engine))
+
+    def last_offload_ms(self) -> float:
+        """Device time of the last finished offloaded step, first H2D to last D2H."""
+        ms = ctypes.c_float()
+        _C.check("ft_offload_elapsed_ms", self._lib.ft_offload_elapsed_ms(self._offload_engine(), ctypes.byref(ms)))
+        return float(ms.value)
+
+
+class FlexTrainAdam(FlexTrainOptimizer):
+    """User-facing Adam: creates the step engine, then groups parameters
+    (reference ``flextrain/ops/adam/__init__.py:10-34``). Extra keyword arguments go to
+    ``FlexTrainOptimizer`` (dtypes, ``offload``, ``loss_scaler``, ``max_grad_norm``...)."""
+
+    def __init__(
+        self,
+        param_groups: List[Dict],
+        lr=1e-3,
+        bias_correction=True,
+        betas=(0.9, 0.999),
+        eps=1e-8,
+        weight_decay=0.01,
+        amsgrad=False,
+        adamw_mode=True,
+        **optimizer_kwargs,
+    ):
+        self.cpu_optimizer = FlexTrainCPUAdam(
+            lr=lr, bias_correction=bias_correction, betas=betas, eps=eps,
+            weight_decay=weight_decay, amsgrad=amsgrad, adamw_mode=adamw_mode,
+        )
+        super().__init__(param_groups=param_groups, **optimizer_kwargs)

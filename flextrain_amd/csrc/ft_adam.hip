@@ -1,0 +1,392 @@
+// ft_adam.hip -- resident optimizer step, gradient statistics and the registry behind the C ABI.
+//
+// Replaces the native half of the reference's optimizer step:
+//   flextrain/ops/csrc/adam/cpu_adam.cpp:8-16        (the four exported functions)
+//   flextrain/ops/csrc/adam/cpu_adam_impl.cpp:143-302 (registry, marshalling, work partition)
+//   flextrain/ops/csrc/includes/cpu_adam.h:67-102     (host scalars)
+// The arithmetic itself lives in ft_kernels.hpp.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include <cmath>
+#include <mutex>
+#include <unordered_map>
+
+#include "ft_internal.hpp"
+#include "ft_kernels.hpp"
+
+#ifndef FT_ADAM_BLOCK
+#define FT_ADAM_BLOCK 256
+#endif
+#ifndef FT_ADAM_UNROLL
+#define FT_ADAM_UNROLL 2
+#endif
+#ifndef FT_ADAM_NT_LD
+#define FT_ADAM_NT_LD true
+#endif
+#ifndef FT_ADAM_NT_ST
+#define FT_ADAM_NT_ST true
+#endif
+#ifndef FT_ADAM_BLOCKS_PER_CU
+#define FT_ADAM_BLOCKS_PER_CU 8
+#endif
+#ifndef FT_STATS_BLOCK
+#define FT_STATS_BLOCK 256
+#endif
+#ifndef FT_STATS_UNROLL
+#define FT_STATS_UNROLL 4
+#endif
+#ifndef FT_STATS_BLOCKS_PER_CU
+#define FT_STATS_BLOCKS_PER_CU 8
+#endif
+
+namespace {
+
+thread_local std::string t_last_error;
+
+std::mutex g_mu;
+std::unordered_map<int, fth::AdamObject> g_adams;
+std::unordered_map<int, int> g_cu_count;      // device -> compute units
+std::unordered_map<int, void*> g_stats_ws;    // device -> library-owned statistics scratch
+int g_adam_blocks_per_cu = FT_ADAM_BLOCKS_PER_CU;
+int g_stats_blocks_per_cu = FT_STATS_BLOCKS_PER_CU;
+
+constexpr int kMaxStatsBlocks = 8192;
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+inline size_t elem_size(int dt) { return dt == FT_F32 ? 4 : 2; }
+inline bool valid_dtype(int dt) { return dt == FT_F32 || dt == FT_F16 || dt == FT_BF16; }
+
+}  // namespace
+
+namespace fth {
+
+int fail(int code, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    t_last_error = buf;
+    return code;
+}
+
+int find_adam(int id, AdamObject* out)
+{
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_adams.find(id);
+    if (it == g_adams.end()) return fail(FT_ENOENT, "no optimizer with id %d (ft_adam_create first)", id);
+    *out = it->second;
+    return FT_OK;
+}
+
+int cu_count()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_cu_count.find(dev);
+    if (it != g_cu_count.end()) return it->second;
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    g_cu_count[dev] = n;
+    return n;
+}
+
+ftk::AdamConsts make_consts(uint64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
+                            bool bias_correction, bool adamw_mode, float grad_mult)
+{
+    // beta^t: the reference calls std::pow(float, size_t), i.e. the double overload, and stores the
+    // result in a float member (cpu_adam.h:73-74). Everything after that is float arithmetic.
+    const float b1t = static_cast<float>(std::pow(static_cast<double>(beta1), static_cast<double>(step)));
+    const float b2t = static_cast<float>(std::pow(static_cast<double>(beta2), static_cast<double>(step)));
+    float bias1 = 1.0f, bias2 = 1.0f;
+    if (bias_correction) {
+        bias1 = 1.0f - b1t;
+        bias2 = 1.0f / sqrtf(1.0f - b2t);
+    }
+    ftk::AdamConsts c;
+    c.beta1 = beta1;
+    c.beta2 = beta2;
+    c.omb1 = 1.0f - beta1;
+    c.omb2 = 1.0f - beta2;
+    c.bias2 = bias2;
+    c.eps = eps;
+    c.step_size = (-1.0f * lr) / bias1;
+    c.wd_mode = 0;
+    c.wd_coef = 0.0f;
+    if (weight_decay > 0.0f) {
+        c.wd_mode = adamw_mode ? 1 : 2;
+        c.wd_coef = adamw_mode ? (-1.0f * lr) * weight_decay : weight_decay;
+    }
+    c.grad_mult = grad_mult;
+    return c;
+}
+
+namespace {
+
+template <int GT, int HT>
+int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, float* v, void* h, size_t n,
+                 const ft_step_control_t* ctl, hipStream_t stream)
+{
+    constexpr size_t gsz = (GT == FT_F32) ? 4 : 2;
+    const char* gb = reinterpret_cast<const char*>(g);
+    char* mb = reinterpret_cast<char*>(m);
+    char* vb = reinterpret_cast<char*>(v);
+    char* hb = reinterpret_cast<char*>(h);
+
+    // Elements before the first 16-byte boundary of p. The vector body needs every array to reach
+    // its own vector alignment after the same number of elements; flat buffers sliced at a common
+    // element offset (the reference's StepContext views, flextrain/param_group.py:196-199) do.
+    size_t head = ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4;
+    if (head > n) head = n;
+    const bool vec_ok = aligned(mb + head * 4, 16) && aligned(vb + head * 4, 16) &&
+                        aligned(gb + head * gsz, gsz * 4) && (h == nullptr || aligned(hb + head * 2, 8));
+    const size_t nvec = vec_ok ? (n - head) / 4 : 0;
+    const size_t body = nvec * 4;
+
+    auto scalar_part = [&](size_t off, size_t cnt) -> int {
+        if (cnt == 0) return FT_OK;
+        ftk::AdamArgs a;
+        a.p = p + off;
+        a.g = gb + off * gsz;
+        a.m = m + off;
+        a.v = v + off;
+        a.h = h ? hb + off * 2 : nullptr;
+        a.ctl = ctl;
+        a.n = cnt;
+        a.c = c;
+        size_t blocks = (cnt + 255) / 256;
+        const size_t cap = static_cast<size_t>(cu_count()) * 16;
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL((ftk::adam_scalar_kernel<GT, HT>), dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                           stream, a);
+        FT_HIP(hipGetLastError());
+        return FT_OK;
+    };
+
+    if (!vec_ok) return scalar_part(0, n);
+
+    if (nvec > 0) {
+        ftk::AdamArgs a;
+        a.p = p + head;
+        a.g = gb + head * gsz;
+        a.m = m + head;
+        a.v = v + head;
+        a.h = h ? hb + head * 2 : nullptr;
+        a.ctl = ctl;
+        a.n = nvec;
+        a.c = c;
+        constexpr size_t kTile = static_cast<size_t>(FT_ADAM_BLOCK) * FT_ADAM_UNROLL;
+        size_t blocks = (nvec + kTile - 1) / kTile;
+        const size_t cap = static_cast<size_t>(cu_count()) * static_cast<size_t>(g_adam_blocks_per_cu);
+        if (blocks > cap) blocks = cap;
+        hipLaunchKernelGGL(
+            (ftk::adam_vec_kernel<GT, HT, FT_ADAM_BLOCK, FT_ADAM_UNROLL, FT_ADAM_NT_LD, FT_ADAM_NT_ST>),
+            dim3(static_cast<unsigned>(blocks)), dim3(FT_ADAM_BLOCK), 0, stream, a);
+        FT_HIP(hipGetLastError());
+    }
+    int rc = scalar_part(0, head);
+    if (rc != FT_OK) return rc;
+    return scalar_part(head + body, n - head - body);
+}
+
+template <int GT>
+int launch_g(const ftk::AdamConsts& c, float* p, const void* g, float* m, float* v, void* h, int half_dtype,
+             size_t n, const ft_step_control_t* ctl, hipStream_t stream)
+{
+    if (h == nullptr) return launch_typed<GT, -1>(c, p, g, m, v, nullptr, n, ctl, stream);
+    if (half_dtype == FT_F16) return launch_typed<GT, FT_F16>(c, p, g, m, v, h, n, ctl, stream);
+    return launch_typed<GT, FT_BF16>(c, p, g, m, v, h, n, ctl, stream);
+}
+
+}  // namespace
+
+int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, float* m, float* v,
+                void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream)
+{
+    if (n == 0) return FT_OK;
+    if (!p || !g || !m || !v) return fail(FT_EINVAL, "params, grads, exp_avg and exp_avg_sq must not be NULL");
+    if (!valid_dtype(g_dtype)) return fail(FT_EINVAL, "unknown gradient dtype code %d", g_dtype);
+    if (half_out && half_dtype != FT_F16 && half_dtype != FT_BF16)
+        return fail(FT_EINVAL, "low-precision copy must be FT_F16 or FT_BF16, got %d", half_dtype);
+    if (!aligned(p, 4) || !aligned(m, 4) || !aligned(v, 4) || !aligned(g, elem_size(g_dtype)) ||
+        (half_out && !aligned(half_out, 2)))
+        return fail(FT_EALIGN, "a pointer is not aligned to its element size");
+    if (ctl && !aligned(ctl, 16)) return fail(FT_EALIGN, "ft_step_control_t must be 16-byte aligned");
+    switch (g_dtype) {
+        case FT_F32: return launch_g<FT_F32>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream);
+        case FT_F16: return launch_g<FT_F16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream);
+        default: return launch_g<FT_BF16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream);
+    }
+}
+
+}  // namespace fth
+
+// ================================================================================================
+// C ABI
+// ================================================================================================
+extern "C" {
+
+const char* ft_last_error(void) { return t_last_error.c_str(); }
+
+int ft_abi_version(void) { return 1; }
+
+int ft_device_count(void)
+{
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fth::fail(FT_EHIP, "hipGetDeviceCount failed: %s", hipGetErrorString(e));
+    }
+    return n;
+}
+
+int ft_adam_create(int id, float lr, float beta1, float beta2, float eps, float weight_decay, int adamw_mode,
+                   int should_log)
+{
+    fth::AdamObject o{lr, beta1, beta2, eps, weight_decay, adamw_mode != 0};
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        g_adams[id] = o;
+    }
+    if (should_log) {
+        printf("Adam Optimizer #%d is created with gfx950 HIP arithmetic capability.\n", id);
+        printf("Config: alpha=%f, betas=(%f, %f), weight_decay=%f, adam_w=%d\n", lr, beta1, beta2, weight_decay,
+               adamw_mode != 0);
+        fflush(stdout);
+    }
+    return FT_OK;
+}
+
+int ft_adam_destroy(int id)
+{
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_adams.erase(id);
+    return FT_OK;
+}
+
+int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
+                 int bias_correction, float grad_mult, void* p, const void* g, int g_dtype, void* m, void* v,
+                 void* half_out, int half_dtype, size_t n, const void* ctl, void* stream)
+{
+    fth::AdamObject o;
+    int rc = fth::find_adam(id, &o);
+    if (rc != FT_OK) return rc;
+    const ftk::AdamConsts c =
+        fth::make_consts(step, lr, beta1, beta2, eps, weight_decay, bias_correction != 0, o.adamw_mode, grad_mult);
+    return fth::launch_adam(c, static_cast<float*>(p), g, g_dtype, static_cast<float*>(m), static_cast<float*>(v),
+                            half_out, half_dtype, n, static_cast<const ft_step_control_t*>(ctl),
+                            static_cast<hipStream_t>(stream));
+}
+
+size_t ft_grad_stats_workspace_bytes(void) { return sizeof(ftk::StatsPartial) * kMaxStatsBlocks; }
+
+int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate, void* workspace,
+                  size_t workspace_bytes, void* stream_)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (!out) return fth::fail(FT_EINVAL, "out must not be NULL");
+    if (!aligned(out, 16)) return fth::fail(FT_EALIGN, "ft_grad_stats_t must be 16-byte aligned");
+    if (!valid_dtype(g_dtype)) return fth::fail(FT_EINVAL, "unknown gradient dtype code %d", g_dtype);
+    if (n > 0 && !g) return fth::fail(FT_EINVAL, "g must not be NULL");
+    if (n > 0 && !aligned(g, elem_size(g_dtype))) return fth::fail(FT_EALIGN, "g is not aligned to its element size");
+
+    ftk::StatsPartial* parts = static_cast<ftk::StatsPartial*>(workspace);
+    if (parts) {
+        if (workspace_bytes < ft_grad_stats_workspace_bytes())
+            return fth::fail(FT_EINVAL, "workspace of %zu bytes is smaller than ft_grad_stats_workspace_bytes()",
+                             workspace_bytes);
+        if (!aligned(parts, 16)) return fth::fail(FT_EALIGN, "workspace must be 16-byte aligned");
+    } else {
+        int dev = 0;
+        FT_HIP(hipGetDevice(&dev));
+        std::lock_guard<std::mutex> lk(g_mu);
+        auto it = g_stats_ws.find(dev);
+        if (it == g_stats_ws.end()) {
+            void* w = nullptr;
+            FT_HIP(hipMalloc(&w, ft_grad_stats_workspace_bytes()));
+            g_stats_ws[dev] = w;
+            parts = static_cast<ftk::StatsPartial*>(w);
+        } else {
+            parts = static_cast<ftk::StatsPartial*>(it->second);
+        }
+    }
+
+    const size_t esz = elem_size(g_dtype);
+    const size_t per_unit = 16 / esz;
+    size_t head = 0;
+    if (n > 0) {
+        head = ((16 - (reinterpret_cast<uintptr_t>(g) & 15)) & 15) / esz;
+        if (head > n) head = n;
+    }
+    const size_t nvec = (n - head) / per_unit;
+    const size_t tail_begin = head + nvec * per_unit;
+    int blocks = 0;
+    if (nvec > 0) {
+        constexpr size_t kTile = static_cast<size_t>(FT_STATS_BLOCK) * FT_STATS_UNROLL;
+        size_t b = (nvec + kTile - 1) / kTile;
+        size_t cap = static_cast<size_t>(fth::cu_count()) * static_cast<size_t>(g_stats_blocks_per_cu);
+        if (cap > static_cast<size_t>(kMaxStatsBlocks)) cap = kMaxStatsBlocks;
+        if (b > cap) b = cap;
+        blocks = static_cast<int>(b);
+        const ftk::u32x4* gv = reinterpret_cast<const ftk::u32x4*>(static_cast<const char*>(g) + head * esz);
+        switch (g_dtype) {
+            case FT_F32:
+                hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F32, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts);
+                break;
+            case FT_F16:
+                hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts);
+                break;
+            default:
+                hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_BF16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts);
+                break;
+        }
+        FT_HIP(hipGetLastError());
+    }
+    ft_grad_stats_t* o = static_cast<ft_grad_stats_t*>(out);
+    switch (g_dtype) {
+        case FT_F32:
+            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
+                               head, tail_begin, n, pre_mult, o, accumulate);
+            break;
+        case FT_F16:
+            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
+                               head, tail_begin, n, pre_mult, o, accumulate);
+            break;
+        default:
+            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_BF16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
+                               head, tail_begin, n, pre_mult, o, accumulate);
+            break;
+    }
+    FT_HIP(hipGetLastError());
+    return FT_OK;
+}
+
+int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ctl_out, void* stream)
+{
+    if (!stats || !ctl_out) return fth::fail(FT_EINVAL, "stats and ctl_out must not be NULL");
+    if (!aligned(stats, 16) || !aligned(ctl_out, 16))
+        return fth::fail(FT_EALIGN, "stats and ctl_out must be 16-byte aligned");
+    hipLaunchKernelGGL(ftk::grad_control_kernel, dim3(1), dim3(1), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const ft_grad_stats_t*>(stats), inv_scale, max_norm,
+                       static_cast<ft_step_control_t*>(ctl_out));
+    FT_HIP(hipGetLastError());
+    return FT_OK;
+}
+
+int ft_set_launch_tuning(int adam_blocks_per_cu, int stats_blocks_per_cu)
+{
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_adam_blocks_per_cu = adam_blocks_per_cu > 0 ? adam_blocks_per_cu : FT_ADAM_BLOCKS_PER_CU;
+    g_stats_blocks_per_cu = stats_blocks_per_cu > 0 ? stats_blocks_per_cu : FT_STATS_BLOCKS_PER_CU;
+    return FT_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,43 @@
+// ft_internal.hpp -- helpers shared by the translation units of libftadam.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "ft_adam.h"
+#include "ft_types.hpp"
+
+namespace fth {
+
+// Records `msg` as the calling thread's last error and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define FT_HIP(call)                                                                      \
+    do {                                                                                  \
+        hipError_t _e = (call);                                                           \
+        if (_e != hipSuccess)                                                             \
+            return ::fth::fail(FT_EHIP, "%s failed: %s (%s:%d)", #call, hipGetErrorString(_e), \
+                               __FILE__, __LINE__);                                       \
+    } while (0)
+
+struct AdamObject {
+    float lr, beta1, beta2, eps, weight_decay;
+    bool adamw_mode;
+};
+
+// Looks the optimizer up; returns FT_ENOENT if absent.
+int find_adam(int id, AdamObject* out);
+
+// Host scalars of one step (cpu_adam.h:67-102,148-166 of the reference).
+ftk::AdamConsts make_consts(uint64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
+                            bool bias_correction, bool adamw_mode, float grad_mult);
+
+// Validates and launches the update over n elements on `stream` (device of the current context).
+int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, float* m, float* v,
+                void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream);
+
+int cu_count();  // compute units of the current device (cached)
+
+}  // namespace fth

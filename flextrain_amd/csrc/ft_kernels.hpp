@@ -1,0 +1,422 @@
+// ft_kernels.hpp -- gfx950 device code of the optimizer-step hot path.
+//
+// Two kernels carry the traffic:
+//   adam_vec_kernel   fused unscale/clip multiply + Adam/AdamW + low-precision recast. One pass:
+//                     reads p, m, v (fp32) and g (fp32/fp16/bf16), writes p, m, v and optionally
+//                     the 16-bit copy. HBM-bound: 28 bytes per element with 16-bit g and copy.
+//   grad_stats_kernel one read of g: inf/nan count and sum of squares (2 or 4 bytes per element).
+//
+// Arithmetic contract of adam_element(): one IEEE-754 round-to-nearest fp32 operation per
+// statement, in the order of the reference's vector loop
+// (flextrain/ops/csrc/includes/cpu_adam.h:188-205). The translation unit must be compiled with
+// -ffp-contract=off; fused multiply-adds appear only where written as __builtin_fmaf. Division
+// and square root are the correctly rounded expansions hipcc emits by default.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ft_adam.h"
+#include "ft_types.hpp"
+
+namespace ftk {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ void adam_element(float& p, float g, float& m, float& v, const AdamConsts& c)
+{
+    g = g * c.grad_mult;
+    if (c.wd_mode == 2) g = __builtin_fmaf(p, c.wd_coef, g);
+    float mi = m * c.beta1;
+    mi = __builtin_fmaf(g, c.omb1, mi);
+    float vi = v * c.beta2;
+    const float g2 = g * g;
+    vi = __builtin_fmaf(g2, c.omb2, vi);
+    float d = __builtin_sqrtf(vi);
+    d = __builtin_fmaf(d, c.bias2, c.eps);
+    const float u = mi / d;
+    float pi = p;
+    if (c.wd_mode == 1) pi = __builtin_fmaf(pi, c.wd_coef, pi);
+    pi = __builtin_fmaf(u, c.step_size, pi);
+    // The new value is materialised in a register before any narrowing conversion, so that the
+    // 16-bit copy is the rounding of the stored fp32 value and never a mixed-precision fma.
+    asm volatile("" : "+v"(pi));
+    p = pi;
+    m = mi;
+    v = vi;
+}
+
+// Four consecutive elements held in vector registers.
+__device__ __forceinline__ void adam_unit(f32x4& p, const f32x4& g, f32x4& m, f32x4& v, const AdamConsts& c)
+{
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float pk = p[k], mk = m[k], vk = v[k];
+        adam_element(pk, g[k], mk, vk, c);
+        p[k] = pk;
+        m[k] = mk;
+        v[k] = vk;
+    }
+}
+
+// ---- 16-bit <-> 32-bit helpers ------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ float half_to_float(uint32_t bits16);
+template <>
+__device__ __forceinline__ float half_to_float<FT_BF16>(uint32_t b)
+{
+    return __builtin_bit_cast(float, b << 16);
+}
+template <>
+__device__ __forceinline__ float half_to_float<FT_F16>(uint32_t b)
+{
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <>
+__device__ __forceinline__ uint32_t pack2<FT_BF16>(float lo, float hi)
+{
+    f32x2 x = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+}
+template <>
+__device__ __forceinline__ uint32_t pack2<FT_F16>(float lo, float hi)
+{
+    f32x2 x = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+}
+
+template <bool NT, typename T>
+__device__ __forceinline__ T ld(const T* p)
+{
+    if constexpr (NT)
+        return __builtin_nontemporal_load(p);
+    else
+        return *p;
+}
+template <bool NT, typename T>
+__device__ __forceinline__ void st(T* p, T x)
+{
+    if constexpr (NT)
+        __builtin_nontemporal_store(x, p);
+    else
+        *p = x;
+}
+
+// Gradient unit = 4 consecutive elements.
+template <int GT, bool NT>
+__device__ __forceinline__ f32x4 load_g4(const void* g, uint64_t unit)
+{
+    if constexpr (GT == FT_F32) {
+        return ld<NT>(reinterpret_cast<const f32x4*>(g) + unit);
+    } else {
+        const u32x2 w = ld<NT>(reinterpret_cast<const u32x2*>(g) + unit);
+        f32x4 r;
+        r.x = half_to_float<GT>(w.x & 0xffffu);
+        r.y = half_to_float<GT>(w.x >> 16);
+        r.z = half_to_float<GT>(w.y & 0xffffu);
+        r.w = half_to_float<GT>(w.y >> 16);
+        return r;
+    }
+}
+
+template <int HT, bool NT>
+__device__ __forceinline__ void store_h4(void* h, uint64_t unit, f32x4 p)
+{
+    if constexpr (HT == FT_F16 || HT == FT_BF16) {
+        u32x2 w;
+        w.x = pack2<HT>(p.x, p.y);
+        w.y = pack2<HT>(p.z, p.w);
+        st<NT>(reinterpret_cast<u32x2*>(h) + unit, w);
+    }
+}
+
+// HT == -1: no low-precision copy.
+template <int GT, int HT, int BLOCK, int UNROLL, bool NT_LD, bool NT_ST>
+__global__ __launch_bounds__(BLOCK) void adam_vec_kernel(AdamArgs a)
+{
+    AdamConsts c = a.c;
+    if (a.ctl) {  // wave-uniform: one decision per step
+        if (a.ctl->skip) return;
+        c.grad_mult = a.ctl->grad_mult;
+    }
+    const uint64_t nvec = a.n;
+    constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
+    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+    f32x4* __restrict__ P = reinterpret_cast<f32x4*>(a.p);
+    f32x4* __restrict__ M = reinterpret_cast<f32x4*>(a.m);
+    f32x4* __restrict__ V = reinterpret_cast<f32x4*>(a.v);
+
+    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const uint64_t base = tile * kTile + threadIdx.x;
+        f32x4 p[UNROLL], m[UNROLL], v[UNROLL], g[UNROLL];
+        if ((tile + 1) * kTile <= nvec) {
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint64_t i = base + (uint64_t)u * BLOCK;
+                g[u] = load_g4<GT, NT_LD>(a.g, i);
+                p[u] = ld<NT_LD>(P + i);
+                m[u] = ld<NT_LD>(M + i);
+                v[u] = ld<NT_LD>(V + i);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                adam_unit(p[u], g[u], m[u], v[u], c);
+            }
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint64_t i = base + (uint64_t)u * BLOCK;
+                st<NT_ST>(P + i, p[u]);
+                st<NT_ST>(M + i, m[u]);
+                st<NT_ST>(V + i, v[u]);
+                store_h4<HT, NT_ST>(a.h, i, p[u]);
+            }
+        } else {  // last, partial tile
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint64_t i = base + (uint64_t)u * BLOCK;
+                if (i >= nvec) break;
+                f32x4 gg = load_g4<GT, false>(a.g, i);
+                f32x4 pp = P[i], mm = M[i], vv = V[i];
+                adam_unit(pp, gg, mm, vv, c);
+                P[i] = pp;
+                M[i] = mm;
+                V[i] = vv;
+                store_h4<HT, false>(a.h, i, pp);
+            }
+        }
+    }
+}
+
+// Element-at-a-time kernel for heads, tails and arrays whose alignments disagree. a.n counts
+// elements. Same arithmetic, so the result of an element never depends on which kernel took it.
+template <int GT, int HT>
+__global__ __launch_bounds__(256) void adam_scalar_kernel(AdamArgs a)
+{
+    AdamConsts c = a.c;
+    if (a.ctl) {
+        if (a.ctl->skip) return;
+        c.grad_mult = a.ctl->grad_mult;
+    }
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += stride) {
+        float g;
+        if constexpr (GT == FT_F32)
+            g = reinterpret_cast<const float*>(a.g)[i];
+        else
+            g = half_to_float<GT>(reinterpret_cast<const uint16_t*>(a.g)[i]);
+        float p = a.p[i], m = a.m[i], v = a.v[i];
+        adam_element(p, g, m, v, c);
+        a.p[i] = p;
+        a.m[i] = m;
+        a.v[i] = v;
+        if constexpr (HT == FT_F16 || HT == FT_BF16)
+            reinterpret_cast<uint16_t*>(a.h)[i] = (uint16_t)(pack2<HT>(p, 0.0f) & 0xffffu);
+    }
+}
+
+// ---- reductions ----------------------------------------------------------------------------
+// Sum across the 64 lanes of a wavefront with DPP lane permutes (no LDS): xor-1 and xor-2 inside
+// each quad, then mirror inside half rows and rows; every lane of a 16-lane row then holds the
+// row total, and the four row totals are read with v_readlane and added in a fixed order.
+__device__ __forceinline__ float wave_sum(float x)
+{
+    int xi;
+    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false);  // quad_perm:[1,0,3,2]
+    x += __builtin_bit_cast(float, xi);
+    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false);  // quad_perm:[2,3,0,1]
+    x += __builtin_bit_cast(float, xi);
+    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false);  // row_half_mirror
+    x += __builtin_bit_cast(float, xi);
+    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false);  // row_mirror
+    x += __builtin_bit_cast(float, xi);
+    const int b = __builtin_bit_cast(int, x);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
+    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t x)
+{
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x4E, 0xF, 0xF, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x141, 0xF, 0xF, false);
+    x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0x140, 0xF, 0xF, false);
+    return (uint32_t)__builtin_amdgcn_readlane((int)x, 0) + (uint32_t)__builtin_amdgcn_readlane((int)x, 16) +
+           (uint32_t)__builtin_amdgcn_readlane((int)x, 32) + (uint32_t)__builtin_amdgcn_readlane((int)x, 48);
+}
+
+struct StatsPartial {
+    double sumsq;
+    uint64_t nonfinite;
+};
+
+// One 16-byte load = 8 sixteen-bit or 4 thirty-two-bit gradient elements.
+template <int GT>
+__device__ __forceinline__ void stats_accumulate(u32x4 w, float pre_mult, float (&acc)[4], uint32_t& bad)
+{
+    if constexpr (GT == FT_F32) {
+        const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const bool nf = (ws[k] & 0x7f800000u) == 0x7f800000u;
+            const float x = __builtin_bit_cast(float, ws[k]) * pre_mult;
+            bad += nf ? 1u : 0u;
+            acc[k] = __builtin_fmaf(nf ? 0.0f : x, nf ? 0.0f : x, acc[k]);
+        }
+    } else {
+        constexpr uint32_t kExp = (GT == FT_BF16) ? 0x7f80u : 0x7c00u;
+        const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t lo = ws[k] & 0xffffu, hi = ws[k] >> 16;
+            const bool nlo = (lo & kExp) == kExp, nhi = (hi & kExp) == kExp;
+            const float xlo = half_to_float<GT>(lo) * pre_mult;
+            const float xhi = half_to_float<GT>(hi) * pre_mult;
+            bad += (nlo ? 1u : 0u) + (nhi ? 1u : 0u);
+            acc[k] = __builtin_fmaf(nlo ? 0.0f : xlo, nlo ? 0.0f : xlo, acc[k]);
+            acc[k] = __builtin_fmaf(nhi ? 0.0f : xhi, nhi ? 0.0f : xhi, acc[k]);
+        }
+    }
+}
+
+// Stage 1: every block writes one StatsPartial. nvec = number of 16-byte units; the caller
+// handles the elements outside [0, nvec*per_unit) in grad_stats_final_kernel.
+template <int GT, int BLOCK, int UNROLL>
+__global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restrict__ g, uint64_t nvec,
+                                                           float pre_mult, StatsPartial* __restrict__ partials)
+{
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    uint32_t bad = 0;
+    constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
+    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const uint64_t base = tile * kTile + threadIdx.x;
+        if ((tile + 1) * kTile <= nvec) {
+            u32x4 w[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) w[u] = __builtin_nontemporal_load(g + base + (uint64_t)u * BLOCK);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(w[u], pre_mult, acc, bad);
+        } else {
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint64_t i = base + (uint64_t)u * BLOCK;
+                if (i >= nvec) break;
+                stats_accumulate<GT>(g[i], pre_mult, acc, bad);
+            }
+        }
+    }
+    const float t = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+    const uint32_t tb = wave_sum_u32(bad);
+
+    constexpr int kWaves = BLOCK / kWave;
+    __shared__ float s_sum[kWaves];
+    __shared__ uint32_t s_bad[kWaves];
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        s_sum[wave] = t;
+        s_bad[wave] = tb;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double s = 0.0;
+        uint64_t b = 0;
+#pragma unroll
+        for (int k = 0; k < kWaves; ++k) {
+            s += (double)s_sum[k];
+            b += s_bad[k];
+        }
+        partials[blockIdx.x].sumsq = s;
+        partials[blockIdx.x].nonfinite = b;
+    }
+}
+
+// Stage 2 (one block of 256): adds the block partials in a fixed tree order, then the up to
+// `edge` elements before/after the vector body one by one, and writes or accumulates the result.
+template <int GT>
+__global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartial* __restrict__ partials,
+                                                               int nparts, const void* g, uint64_t head,
+                                                               uint64_t tail_begin, uint64_t n, float pre_mult,
+                                                               ft_grad_stats_t* out, int accumulate)
+{
+    __shared__ double s_sum[256];
+    __shared__ uint64_t s_bad[256];
+    double s = 0.0;
+    uint64_t b = 0;
+    for (int i = threadIdx.x; i < nparts; i += 256) {
+        s += partials[i].sumsq;
+        b += partials[i].nonfinite;
+    }
+    s_sum[threadIdx.x] = s;
+    s_bad[threadIdx.x] = b;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
+            s_bad[threadIdx.x] += s_bad[threadIdx.x + w];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        s = s_sum[0];
+        b = s_bad[0];
+        for (uint64_t i = 0; i < n; ++i) {
+            if (i == head) i = tail_begin;  // skip the vector body
+            if (i >= n) break;
+            float x;
+            bool nf;
+            if constexpr (GT == FT_F32) {
+                const uint32_t w = reinterpret_cast<const uint32_t*>(g)[i];
+                nf = (w & 0x7f800000u) == 0x7f800000u;
+                x = __builtin_bit_cast(float, w);
+            } else {
+                constexpr uint32_t kExp = (GT == FT_BF16) ? 0x7f80u : 0x7c00u;
+                const uint32_t w = reinterpret_cast<const uint16_t*>(g)[i];
+                nf = (w & kExp) == kExp;
+                x = half_to_float<GT>(w);
+            }
+            if (nf) {
+                b += 1;
+            } else {
+                const float u = x * pre_mult;
+                s += (double)u * (double)u;
+            }
+        }
+        if (accumulate) {
+            out->sumsq += s;
+            out->nonfinite += b;
+        } else {
+            out->sumsq = s;
+            out->nonfinite = b;
+        }
+    }
+}
+
+__global__ void grad_control_kernel(const ft_grad_stats_t* stats, float inv_scale, float max_norm,
+                                    ft_step_control_t* ctl)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const double norm = __builtin_sqrt(stats->sumsq);
+    double coef = 1.0;
+    if (max_norm > 0.0f) {
+        coef = (double)max_norm / (norm + 1e-6);
+        if (!(coef < 1.0)) coef = 1.0;
+    }
+    const float clip = (float)coef;
+    ctl->skip = stats->nonfinite != 0 ? 1u : 0u;
+    ctl->grad_mult = clip * inv_scale;
+    ctl->grad_norm = (float)norm;
+    ctl->clip_coef = clip;
+}
+
+}  // namespace ftk

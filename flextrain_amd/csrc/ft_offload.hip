@@ -1,0 +1,333 @@
+// ft_offload.hip -- pinned host memory, the chunked host<->HBM optimizer pipeline and the link probe.
+//
+// Replaces, for state that lives in pinned host DRAM, the reference's arrangement of
+//   flextrain/memory/__init__.py:240-248  RotateContainer (rotating buffer sets)
+//   flextrain/memory/__init__.py:366-395  FlexTrainDataStream (one side stream, device-wide waits)
+//   flextrain/optimizer.py:244-263        copy grads down, step on the host, copy params up
+// with a three-stage pipeline on three HIP streams. Buffer slots are handed from stage to stage
+// with events, so a copy in one direction, a copy in the other and a kernel run at the same time.
+#include <string.h>
+
+#include <chrono>
+#include <vector>
+
+#include "ft_internal.hpp"
+
+namespace {
+
+struct Slot {
+    float* p = nullptr;
+    float* m = nullptr;
+    float* v = nullptr;
+    void* g = nullptr;  // staging for host-resident gradients (chunk * 4 bytes), lazily allocated
+    void* h = nullptr;  // staging for a host-resident low-precision copy (chunk * 2 bytes), lazy
+    hipEvent_t h2d_done = nullptr, k_done = nullptr, d2h_done = nullptr;
+    bool used = false;
+};
+
+struct Engine {
+    uint32_t magic = 0x46544f45;  // "FTOE"
+    int device = 0;
+    size_t chunk = 0;
+    std::vector<Slot> slots;
+    hipStream_t s_h2d = nullptr, s_k = nullptr, s_d2h = nullptr;
+    hipEvent_t ev_user = nullptr;   // producer stream -> pipeline
+    hipEvent_t ev_begin = nullptr;  // first H2D of the last step
+    hipEvent_t ev_end = nullptr;    // last D2H of the last step
+    hipEvent_t ev_kernels = nullptr;  // last kernel of the last step
+    bool stepped = false;
+};
+
+Engine* as_engine(void* h)
+{
+    Engine* e = static_cast<Engine*>(h);
+    return (e && e->magic == 0x46544f45) ? e : nullptr;
+}
+
+int require_pinned(const void* ptr, const char* what)
+{
+    hipPointerAttribute_t attr;
+    hipError_t err = hipPointerGetAttributes(&attr, ptr);
+    if (err != hipSuccess) {
+        (void)hipGetLastError();
+        return fth::fail(FT_EINVAL, "%s is not pinned host memory (hipPointerGetAttributes: %s)", what,
+                         hipGetErrorString(err));
+    }
+    if (attr.type != hipMemoryTypeHost)
+        return fth::fail(FT_EINVAL, "%s must be pinned host memory (memory type %d)", what, (int)attr.type);
+    return FT_OK;
+}
+
+void destroy_engine(Engine* e)
+{
+    for (Slot& s : e->slots) {
+        if (s.p) (void)hipFree(s.p);
+        if (s.m) (void)hipFree(s.m);
+        if (s.v) (void)hipFree(s.v);
+        if (s.g) (void)hipFree(s.g);
+        if (s.h) (void)hipFree(s.h);
+        if (s.h2d_done) (void)hipEventDestroy(s.h2d_done);
+        if (s.k_done) (void)hipEventDestroy(s.k_done);
+        if (s.d2h_done) (void)hipEventDestroy(s.d2h_done);
+    }
+    if (e->s_h2d) (void)hipStreamDestroy(e->s_h2d);
+    if (e->s_k) (void)hipStreamDestroy(e->s_k);
+    if (e->s_d2h) (void)hipStreamDestroy(e->s_d2h);
+    if (e->ev_user) (void)hipEventDestroy(e->ev_user);
+    if (e->ev_begin) (void)hipEventDestroy(e->ev_begin);
+    if (e->ev_end) (void)hipEventDestroy(e->ev_end);
+    if (e->ev_kernels) (void)hipEventDestroy(e->ev_kernels);
+    e->magic = 0;
+    delete e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ft_pinned_alloc(size_t bytes, void** out)
+{
+    if (!out) return fth::fail(FT_EINVAL, "out must not be NULL");
+    *out = nullptr;
+    if (bytes == 0) return FT_OK;
+    void* p = nullptr;
+    hipError_t e = hipHostMalloc(&p, bytes, hipHostMallocDefault);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fth::fail(FT_ENOMEM, "hipHostMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+    }
+    *out = p;
+    return FT_OK;
+}
+
+int ft_pinned_free(void* ptr)
+{
+    if (!ptr) return FT_OK;
+    FT_HIP(hipHostFree(ptr));
+    return FT_OK;
+}
+
+int ft_offload_create(size_t chunk_elems, int n_slots, void** out_handle)
+{
+    if (!out_handle) return fth::fail(FT_EINVAL, "out_handle must not be NULL");
+    *out_handle = nullptr;
+    if (chunk_elems == 0 || (chunk_elems & 3) != 0)
+        return fth::fail(FT_EINVAL, "chunk_elems must be a positive multiple of 4, got %zu", chunk_elems);
+    if (n_slots < 2 || n_slots > 16) return fth::fail(FT_EINVAL, "n_slots must be in [2, 16], got %d", n_slots);
+
+    Engine* e = new Engine();
+    e->chunk = chunk_elems;
+    e->slots.resize(n_slots);
+    auto bail = [&](hipError_t err, const char* what) {
+        (void)hipGetLastError();
+        destroy_engine(e);
+        return fth::fail(err == hipErrorOutOfMemory ? FT_ENOMEM : FT_EHIP, "%s failed: %s", what,
+                         hipGetErrorString(err));
+    };
+    hipError_t err;
+    if ((err = hipGetDevice(&e->device)) != hipSuccess) return bail(err, "hipGetDevice");
+    if ((err = hipStreamCreateWithFlags(&e->s_h2d, hipStreamNonBlocking)) != hipSuccess) return bail(err, "hipStreamCreate");
+    if ((err = hipStreamCreateWithFlags(&e->s_k, hipStreamNonBlocking)) != hipSuccess) return bail(err, "hipStreamCreate");
+    if ((err = hipStreamCreateWithFlags(&e->s_d2h, hipStreamNonBlocking)) != hipSuccess) return bail(err, "hipStreamCreate");
+    if ((err = hipEventCreateWithFlags(&e->ev_user, hipEventDisableTiming)) != hipSuccess) return bail(err, "hipEventCreate");
+    if ((err = hipEventCreate(&e->ev_begin)) != hipSuccess) return bail(err, "hipEventCreate");
+    if ((err = hipEventCreate(&e->ev_end)) != hipSuccess) return bail(err, "hipEventCreate");
+    if ((err = hipEventCreate(&e->ev_kernels)) != hipSuccess) return bail(err, "hipEventCreate");
+    for (Slot& s : e->slots) {
+        if ((err = hipMalloc(reinterpret_cast<void**>(&s.p), chunk_elems * 4)) != hipSuccess) return bail(err, "hipMalloc");
+        if ((err = hipMalloc(reinterpret_cast<void**>(&s.m), chunk_elems * 4)) != hipSuccess) return bail(err, "hipMalloc");
+        if ((err = hipMalloc(reinterpret_cast<void**>(&s.v), chunk_elems * 4)) != hipSuccess) return bail(err, "hipMalloc");
+        if ((err = hipEventCreateWithFlags(&s.h2d_done, hipEventDisableTiming)) != hipSuccess) return bail(err, "hipEventCreate");
+        if ((err = hipEventCreateWithFlags(&s.k_done, hipEventDisableTiming)) != hipSuccess) return bail(err, "hipEventCreate");
+        if ((err = hipEventCreateWithFlags(&s.d2h_done, hipEventDisableTiming)) != hipSuccess) return bail(err, "hipEventCreate");
+    }
+    *out_handle = e;
+    return FT_OK;
+}
+
+int ft_offload_destroy(void* handle)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    (void)hipStreamSynchronize(e->s_h2d);
+    (void)hipStreamSynchronize(e->s_k);
+    (void)hipStreamSynchronize(e->s_d2h);
+    destroy_engine(e);
+    return FT_OK;
+}
+
+int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, float beta2, float eps,
+                    float weight_decay, int bias_correction, float grad_mult, void* host_p, const void* g,
+                    int g_dtype, int g_on_host, void* host_m, void* host_v, void* half_out, int half_dtype,
+                    int half_on_host, size_t n, const void* ctl, void* stream)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    fth::AdamObject o;
+    int rc = fth::find_adam(id, &o);
+    if (rc != FT_OK) return rc;
+    if (n == 0) return FT_OK;
+    if (!host_p || !host_m || !host_v || !g) return fth::fail(FT_EINVAL, "p, m, v and g must not be NULL");
+    if (g_dtype != FT_F32 && g_dtype != FT_F16 && g_dtype != FT_BF16)
+        return fth::fail(FT_EINVAL, "unknown gradient dtype code %d", g_dtype);
+    if (half_out && half_dtype != FT_F16 && half_dtype != FT_BF16)
+        return fth::fail(FT_EINVAL, "low-precision copy must be FT_F16 or FT_BF16, got %d", half_dtype);
+    if ((rc = require_pinned(host_p, "params")) != FT_OK) return rc;
+    if ((rc = require_pinned(host_m, "exp_avg")) != FT_OK) return rc;
+    if ((rc = require_pinned(host_v, "exp_avg_sq")) != FT_OK) return rc;
+    if (g_on_host && (rc = require_pinned(g, "grads")) != FT_OK) return rc;
+    if (half_out && half_on_host && (rc = require_pinned(half_out, "low-precision copy")) != FT_OK) return rc;
+
+    const size_t gsz = g_dtype == FT_F32 ? 4 : 2;
+    const size_t chunk = e->chunk;
+    if (g_on_host || (half_out && half_on_host)) {
+        for (Slot& s : e->slots) {
+            if (g_on_host && !s.g) FT_HIP(hipMalloc(&s.g, chunk * 4));
+            if (half_out && half_on_host && !s.h) FT_HIP(hipMalloc(&s.h, chunk * 2));
+        }
+    }
+
+    const ftk::AdamConsts c =
+        fth::make_consts(step, lr, beta1, beta2, eps, weight_decay, bias_correction != 0, o.adamw_mode, grad_mult);
+    hipStream_t user = static_cast<hipStream_t>(stream);
+
+    // The pipeline starts after the producer of g/ctl, and after the previous step's last D2H
+    // (a chunk's host copy must be complete before the next step reads it again).
+    FT_HIP(hipEventRecord(e->ev_user, user));
+    FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_user, 0));
+    FT_HIP(hipStreamWaitEvent(e->s_k, e->ev_user, 0));
+    if (e->stepped) FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_end, 0));
+    FT_HIP(hipEventRecord(e->ev_begin, e->s_h2d));
+
+    float* hp = static_cast<float*>(host_p);
+    float* hm = static_cast<float*>(host_m);
+    float* hv = static_cast<float*>(host_v);
+    const char* gb = static_cast<const char*>(g);
+    char* hb = static_cast<char*>(half_out);
+
+    size_t ci = 0;
+    for (size_t off = 0; off < n; off += chunk, ++ci) {
+        const size_t cnt = (n - off < chunk) ? (n - off) : chunk;
+        Slot& s = e->slots[ci % e->slots.size()];
+
+        if (s.used) FT_HIP(hipStreamWaitEvent(e->s_h2d, s.d2h_done, 0));
+        FT_HIP(hipMemcpyAsync(s.p, hp + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
+        FT_HIP(hipMemcpyAsync(s.m, hm + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
+        FT_HIP(hipMemcpyAsync(s.v, hv + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
+        if (g_on_host) FT_HIP(hipMemcpyAsync(s.g, gb + off * gsz, cnt * gsz, hipMemcpyHostToDevice, e->s_h2d));
+        FT_HIP(hipEventRecord(s.h2d_done, e->s_h2d));
+
+        FT_HIP(hipStreamWaitEvent(e->s_k, s.h2d_done, 0));
+        const void* kg = g_on_host ? s.g : static_cast<const void*>(gb + off * gsz);
+        void* kh = nullptr;
+        if (half_out) kh = half_on_host ? s.h : static_cast<void*>(hb + off * 2);
+        rc = fth::launch_adam(c, s.p, kg, g_dtype, s.m, s.v, kh, half_dtype, cnt,
+                              static_cast<const ft_step_control_t*>(ctl), e->s_k);
+        if (rc != FT_OK) return rc;
+        FT_HIP(hipEventRecord(s.k_done, e->s_k));
+
+        FT_HIP(hipStreamWaitEvent(e->s_d2h, s.k_done, 0));
+        FT_HIP(hipMemcpyAsync(hp + off, s.p, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
+        FT_HIP(hipMemcpyAsync(hm + off, s.m, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
+        FT_HIP(hipMemcpyAsync(hv + off, s.v, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
+        if (half_out && half_on_host)
+            FT_HIP(hipMemcpyAsync(hb + off * 2, s.h, cnt * 2, hipMemcpyDeviceToHost, e->s_d2h));
+        FT_HIP(hipEventRecord(s.d2h_done, e->s_d2h));
+        s.used = true;
+    }
+    FT_HIP(hipEventRecord(e->ev_kernels, e->s_k));
+    FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
+    e->stepped = true;
+    // Later work on the producer stream sees the new device-resident low-precision copy (kernels)
+    // and may reuse g (also kernels); waiting for the last D2H as well keeps "step finished" simple.
+    FT_HIP(hipStreamWaitEvent(user, e->ev_kernels, 0));
+    FT_HIP(hipStreamWaitEvent(user, e->ev_end, 0));
+    return FT_OK;
+}
+
+int ft_offload_wait(void* handle)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    if (!e->stepped) return FT_OK;
+    FT_HIP(hipEventSynchronize(e->ev_end));
+    FT_HIP(hipEventSynchronize(e->ev_kernels));
+    return FT_OK;
+}
+
+int ft_offload_elapsed_ms(void* handle, float* out_ms)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    if (!out_ms) return fth::fail(FT_EINVAL, "out_ms must not be NULL");
+    if (!e->stepped) return fth::fail(FT_EINVAL, "no step has been enqueued on this handle");
+    FT_HIP(hipEventSynchronize(e->ev_end));
+    FT_HIP(hipEventElapsedTime(out_ms, e->ev_begin, e->ev_end));
+    return FT_OK;
+}
+
+int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps)
+{
+    if (!out_gbps) return fth::fail(FT_EINVAL, "out_gbps must not be NULL");
+    if (bytes == 0 || iters <= 0 || direction < 0 || direction > 2)
+        return fth::fail(FT_EINVAL, "need bytes > 0, iters > 0 and direction in {0,1,2}");
+    void *h0 = nullptr, *h1 = nullptr, *d0 = nullptr, *d1 = nullptr;
+    hipStream_t s0 = nullptr, s1 = nullptr;
+    int rc = FT_OK;
+    auto cleanup = [&]() {
+        if (s0) (void)hipStreamDestroy(s0);
+        if (s1) (void)hipStreamDestroy(s1);
+        if (h0) (void)hipHostFree(h0);
+        if (h1) (void)hipHostFree(h1);
+        if (d0) (void)hipFree(d0);
+        if (d1) (void)hipFree(d1);
+    };
+#define FT_TRY(call)                                                                             \
+    do {                                                                                         \
+        hipError_t _e = (call);                                                                  \
+        if (_e != hipSuccess) {                                                                  \
+            (void)hipGetLastError();                                                             \
+            rc = fth::fail(FT_EHIP, "%s failed: %s", #call, hipGetErrorString(_e));              \
+            cleanup();                                                                           \
+            return rc;                                                                           \
+        }                                                                                        \
+    } while (0)
+    FT_TRY(hipStreamCreateWithFlags(&s0, hipStreamNonBlocking));
+    FT_TRY(hipStreamCreateWithFlags(&s1, hipStreamNonBlocking));
+    FT_TRY(hipHostMalloc(&h0, bytes, hipHostMallocDefault));
+    FT_TRY(hipMalloc(&d0, bytes));
+    FT_TRY(hipMemsetAsync(d0, 0, bytes, s0));
+    memset(h0, 1, bytes);
+    if (direction == 2) {
+        FT_TRY(hipHostMalloc(&h1, bytes, hipHostMallocDefault));
+        FT_TRY(hipMalloc(&d1, bytes));
+        FT_TRY(hipMemsetAsync(d1, 0, bytes, s1));
+        memset(h1, 1, bytes);
+    }
+    auto enqueue = [&](int k) -> hipError_t {
+        hipError_t err = hipSuccess;
+        for (int i = 0; i < k && err == hipSuccess; ++i) {
+            if (direction == 0 || direction == 2) err = hipMemcpyAsync(d0, h0, bytes, hipMemcpyHostToDevice, s0);
+            if (err != hipSuccess) break;
+            if (direction == 1) err = hipMemcpyAsync(h0, d0, bytes, hipMemcpyDeviceToHost, s0);
+            if (direction == 2) err = hipMemcpyAsync(h1, d1, bytes, hipMemcpyDeviceToHost, s1);
+        }
+        return err;
+    };
+    FT_TRY(enqueue(1));  // warm-up
+    FT_TRY(hipStreamSynchronize(s0));
+    FT_TRY(hipStreamSynchronize(s1));
+    const auto t0 = std::chrono::steady_clock::now();
+    FT_TRY(enqueue(iters));
+    FT_TRY(hipStreamSynchronize(s0));
+    FT_TRY(hipStreamSynchronize(s1));
+    const auto t1 = std::chrono::steady_clock::now();
+#undef FT_TRY
+    const double sec = std::chrono::duration<double>(t1 - t0).count();
+    const double moved = static_cast<double>(bytes) * iters * (direction == 2 ? 2.0 : 1.0);
+    *out_gbps = moved / sec / 1e9;
+    cleanup();
+    return FT_OK;
+}
+
+}  // extern "C"

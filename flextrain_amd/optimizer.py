@@ -1,0 +1,300 @@
+"""Optimizer front end: the reference's ``flextrain/optimizer.py`` surface over GPU kernels.
+
+``FlexTrainCPUOptimizer`` keeps its reference name and abstract methods
+(``flextrain/optimizer.py:24-95``) so that a coordinator written against it keeps working; the
+"CPU" in the name is historical here, the arithmetic runs on the GPU.
+
+``FlexTrainOptimizer`` (reference ``:98-272``) groups parameters, owns the flat buffers of the
+parameters that do not belong to a layer unit, and steps them. What changes against the
+reference is where the data lives: gradients are consumed on the GPU where backward left them
+(no converting D2H copy, ``:253-254``), the master parameters and Adam states are either resident
+in HBM or streamed from pinned host memory, and the low-precision parameters are written by the
+update kernel itself (no converting H2D copy, ``:263``).
+"""
+from __future__ import annotations
+
+from abc import ABC, abstractmethod
+from collections.abc import Iterable
+from typing import Callable, Dict, List, Optional, Union
+
+import torch
+from torch import Tensor
+
+from .param_group import (
+    GroupSegment,
+    ParamGroup,
+    StepContext,
+    create_group_segments,
+    create_step_contexts,
+)
+
+STEP_KEY = "step"
+PARAMS_KEY = "params"
+
+
+class FlexTrainCPUOptimizer(ABC):
+    """Abstract step engine: subclasses implement the arithmetic for one contiguous segment."""
+
+    #: where ``_init_optimizer_states`` and ``profile_step`` place master state:
+    #: "cuda" keeps it resident in HBM, "cpu" keeps it in pinned host memory (streamed step)
+    state_device: str = "cuda"
+
+    @abstractmethod
+    def __init__(self):
+        pass
+
+    @abstractmethod
+    def _init_optimizer_states(self, numel: int, dtype: torch.dtype) -> List[Tensor]:
+        pass
+
+    @abstractmethod
+    def _step(
+        self, param_group: ParamGroup,
+        half_parameter: Optional[Tensor], full_parameter: Tensor,
+        gradient: Tensor, *optimizer_states: Tensor, **extensions
+    ):
+        pass
+
+    @torch.no_grad()
+    def step(self, step_contexts: Union[StepContext, List[StepContext]], **extensions):
+        """Steps every context; contexts without gradient elements are skipped
+        (reference ``flextrain/optimizer.py:44-69``).
+
+        ``extensions`` (``grad_mult``, ``control``) are forwarded to ``_step`` unchanged.
+        """
+        if isinstance(step_contexts, StepContext):
+            step_contexts = [step_contexts]
+        for ctx in step_contexts:
+            if not ctx.gradient.numel():
+                continue
+            self._step(
+                ctx.param_group, ctx.half_parameter, ctx.full_parameter,
+                ctx.gradient, *ctx.optimizer_states, **extensions
+            )
+
+    def _allocate(self, numel: int, dtype: torch.dtype, fill: str) -> Tensor:
+        """A flat buffer on ``state_device`` (pinned when that is the host)."""
+        if self.state_device == "cpu":
+            make = {"zeros": torch.zeros, "empty": torch.empty, "randn": torch.randn}[fill]
+            t = make(numel, dtype=dtype)
+            return t.pin_memory() if numel > 0 else t
+        device = torch.device("cuda", torch.cuda.current_device())
+        make = {"zeros": torch.zeros, "empty": torch.empty, "randn": torch.randn}[fill]
+        return make(numel, dtype=dtype, device=device)
+
+    @torch.no_grad()
+    def profile_step(self, numel: int, device_dtype: torch.dtype, master_dtype: torch.dtype):
+        """One step on private scratch buffers, for throughput probes
+        (reference ``flextrain/optimizer.py:71-95``; driven by ``flextrain/auto_config.py:281-317``).
+        Buffers are created on first use and reused; every call advances a private step counter.
+        """
+        if not hasattr(self, "_param_group"):
+            self._param_group = {STEP_KEY: 0}
+            self._half_parameter = self._allocate(numel, device_dtype, "empty")
+            self._full_parameter = self._allocate(numel, master_dtype, "randn")
+            self._gradient = self._allocate(numel, master_dtype, "randn")
+            self._optimizer_states = self._init_optimizer_states(numel, master_dtype)
+        self._param_group[STEP_KEY] += 1
+        self._step(
+            self._param_group,
+            self._half_parameter, self._full_parameter,
+            self._gradient, *self._optimizer_states
+        )
+
+
+class FlexTrainOptimizer:
+    """Groups parameters for optimisation and steps those that belong to no layer unit.
+
+    Args:
+        param_groups: list of dicts with a ``"params"`` list plus optional hyper-parameters, or a
+            bare iterable of parameters (wrapped into one group).
+        unit_parameter_map: ``{unit_index: object with .paras}`` -- the layer units whose
+            parameters another component steps unit by unit (in the reference this comes from
+            the parameter coordinator, ``flextrain/optimizer.py:131-152``). Default: none, every
+            parameter is stepped here.
+        aligned_unit_numel: padded element count of one unit; the last segment of each unit is
+            stretched to it (``:147-150``).
+        device_dtype / master_dtype / gradacc_dtype: the reference reads these from its global
+            config (``:159-163``); here they are arguments. ``device_dtype`` defaults to the dtype
+            of the first parameter, ``gradacc_dtype`` to ``device_dtype``.
+        offload: keep master parameters and optimizer state in pinned host memory and stream
+            them through the GPU each step, instead of keeping them resident in HBM.
+        loss_scaler: object with ``loss_scale`` and ``update_scale(overflow)``
+            (``flextrain_amd.loss_scaler``); when given, gradients are unscaled by
+            ``1/loss_scale`` inside the update and an inf/nan anywhere skips the step.
+        max_grad_norm: clip the global L2 norm of the unscaled gradients to this value.
+        grad_reduce_fn: called with the flat gradient buffer before anything else (the place of
+            the reference's ``all_reduce(AVG)``, ``:250``); default none (one GPU).
+    """
+
+    cpu_optimizer: FlexTrainCPUOptimizer = None
+
+    def __init__(
+        self,
+        param_groups: List[Dict],
+        *,
+        unit_parameter_map: Optional[Dict[int, object]] = None,
+        aligned_unit_numel: Optional[int] = None,
+        device_dtype: Optional[torch.dtype] = None,
+        master_dtype: torch.dtype = torch.float32,
+        gradacc_dtype: Optional[torch.dtype] = None,
+        offload: bool = False,
+        loss_scaler=None,
+        max_grad_norm: Optional[float] = None,
+        grad_reduce_fn: Optional[Callable[[Tensor], None]] = None,
+    ):
+        assert isinstance(param_groups, Iterable)
+        assert self.cpu_optimizer is not None, "a subclass must create self.cpu_optimizer first"
+        param_groups = list(param_groups)
+        if not all(isinstance(group, dict) for group in param_groups):
+            param_groups = [{PARAMS_KEY: param_groups}]
+        self.param_groups = param_groups
+        self.loss_scaler = loss_scaler
+        self.max_grad_norm = max_grad_norm
+        self._grad_reduce_fn = grad_reduce_fn
+        self._offload = bool(offload)
+        self.cpu_optimizer.state_device = "cpu" if self._offload else "cuda"
+
+        # parameter -> (its group, its position in the caller's order)
+        param_group_map: Dict[Tensor, Dict] = {}
+        param_id_map: Dict[Tensor, int] = {}
+        for group in self.param_groups:
+            assert isinstance(group[PARAMS_KEY], list)
+            for param in group[PARAMS_KEY]:
+                param_group_map[param] = group
+                param_id_map[param] = len(param_id_map)
+
+        # Layer units: record their group segments, and leave their parameters to the caller.
+        self.unit_group_segments: Dict[int, List[GroupSegment]] = {}
+        remaining = dict.fromkeys(param_group_map.keys())
+        for index, unit in (unit_parameter_map or {}).items():
+            paras = list(unit.paras)
+            for p in paras:
+                remaining.pop(p, None)
+            segments = create_group_segments(paras, [param_group_map[p] for p in paras])
+            if aligned_unit_numel is not None and segments:
+                assert segments[-1].end <= aligned_unit_numel
+                segments[-1].end = aligned_unit_numel
+            self.unit_group_segments[index] = segments
+        non_layerwise_params = sorted(remaining.keys(), key=lambda p: param_id_map[p])
+
+        if device_dtype is None:
+            device_dtype = non_layerwise_params[0].dtype if non_layerwise_params else torch.float32
+        if gradacc_dtype is None:
+            gradacc_dtype = device_dtype
+        if master_dtype != torch.float32:
+            raise ValueError("master parameters and optimizer states are fp32 on this path")
+        self._device_dtype, self._master_dtype, self._gradacc_dtype = device_dtype, master_dtype, gradacc_dtype
+        self._gradacc_dtype_incompatible = device_dtype != gradacc_dtype
+
+        device = torch.device("cuda", torch.cuda.current_device())
+        total_numel = sum(p.numel() for p in non_layerwise_params)
+        self._device_para = torch.zeros(total_numel, dtype=device_dtype, device=device)
+        self._device_grad = torch.zeros(total_numel, dtype=device_dtype, device=device)
+        if self._gradacc_dtype_incompatible:
+            self._device_acc_grad = torch.zeros(total_numel, dtype=gradacc_dtype, device=device)
+
+        # Gather the parameters into the flat device buffer (views replace the originals).
+        offset = 0
+        for param in non_layerwise_params:
+            n = param.numel()
+            view = self._device_para[offset:offset + n]
+            view.copy_(param.data.reshape(-1))
+            param.data = view.view(param.shape)
+            offset += n
+
+        # fp32 master copy: resident (aliases the device buffer when that is fp32 already) or
+        # pinned host memory when offloaded.
+        if self._offload:
+            self._master_para = torch.zeros(total_numel, dtype=master_dtype).pin_memory() \
+                if total_numel else torch.zeros(0, dtype=master_dtype)
+            self._master_para.copy_(self._device_para)
+        elif device_dtype == master_dtype:
+            self._master_para = self._device_para
+        else:
+            self._master_para = self._device_para.to(master_dtype)
+        # Wire gradients: backward writes into the flat device buffer (or accumulates into the
+        # wider one through a hook, reference :194-215).
+        self.non_layerwise_master_params: List[torch.nn.Parameter] = []
+        acc_views: List[Tensor] = []
+
+        def _accumulate_into(i: int):
+            def hook(grad: Tensor):
+                acc_views[i] += grad.flatten()
+            return hook
+
+        offset = 0
+        for i, param in enumerate(non_layerwise_params):
+            end = offset + param.numel()
+            self.non_layerwise_master_params.append(torch.nn.Parameter(self._master_para[offset:end]))
+            param.grad = self._device_grad[offset:end].view_as(param)
+            if self._gradacc_dtype_incompatible:
+                acc_views.append(self._device_acc_grad[offset:end])
+                param.register_hook(_accumulate_into(i))
+            offset = end
+
+        grad_buffer = self._device_acc_grad if self._gradacc_dtype_incompatible else self._device_grad
+        self._step_grad = grad_buffer
+        self.non_layerwise_step_contexts = create_step_contexts(
+            group_segments=create_group_segments(
+                non_layerwise_params, [param_group_map[p] for p in non_layerwise_params]),
+            half_parameter=self._device_para if device_dtype != master_dtype else None,
+            full_parameter=self._master_para,
+            gradient=grad_buffer,
+            optimizer_states=self.cpu_optimizer._init_optimizer_states(total_numel, master_dtype),
+        )
+        self.last_step_skipped = False
+        self.last_grad_norm: Optional[float] = None
+
+    @property
+    def optimizer_state_per_element(self) -> int:
+        """Number of optimizer-state tensors per parameter element (2 for Adam)."""
+        return len(self.cpu_optimizer._init_optimizer_states(1, self._master_dtype))
+
+    @property
+    def non_layerwise_numel(self) -> int:
+        return self._device_para.numel()
+
+    def step(self, *args, **kwargs):
+        """Steps the non-layerwise parameters (reference ``flextrain/optimizer.py:244-263``).
+
+        Returns True if the update was applied, False if it was skipped because of inf/nan.
+        """
+        grads = self._step_grad
+        if self._grad_reduce_fn is not None:
+            self._grad_reduce_fn(grads)
+
+        extensions = {}
+        self.last_step_skipped = False
+        if (self.loss_scaler is not None or self.max_grad_norm is not None) and grads.numel():
+            from .loss_scaler import GradientGuard  # local import: keeps module load light
+            if not hasattr(self, "_guard"):
+                self._guard = GradientGuard(device=grads.device)
+            scale = float(self.loss_scaler.loss_scale) if self.loss_scaler is not None else 1.0
+            self._guard.begin()
+            self._guard.add(grads, loss_scale=scale)
+            decision = self._guard.decide(loss_scale=scale, max_grad_norm=self.max_grad_norm)
+            self.last_grad_norm = decision.grad_norm
+            if self.loss_scaler is not None:
+                self.loss_scaler.update_scale(decision.overflow)
+            if decision.overflow:
+                self.last_step_skipped = True
+                self._zero_grads()
+                return False
+            extensions["grad_mult"] = decision.grad_mult
+
+        self.cpu_optimizer.step(self.non_layerwise_step_contexts, **extensions)
+        self._zero_grads()
+        if self._offload and self._device_dtype == self._master_dtype:
+            self._device_para.copy_(self._master_para, non_blocking=True)
+        return True
+
+    def _zero_grads(self):
+        self._device_grad.zero_()
+        if self._gradacc_dtype_incompatible:
+            self._device_acc_grad.zero_()
+
+    def update_states(self):
+        """Advances ``group["step"]`` of every group (reference ``:265-272``)."""
+        for group in self.param_groups:
+            group[STEP_KEY] = group.get(STEP_KEY, 0) + 1

@@ -1,0 +1,164 @@
+/*
+ * ft_adam.h -- C ABI of libftadam.so: the optimizer-step hot path on one MI355X (gfx950).
+ *
+ * Every entry point takes plain pointers and sizes; no framework types cross this boundary.
+ * Device pointers are HIP device (or device-accessible pinned host) addresses owned by the
+ * caller and only borrowed for the call. `stream` is a hipStream_t passed as void* (NULL = the
+ * null stream); all work is enqueued on it and the call returns without waiting unless stated.
+ *
+ * Return value: 0 on success, a negative FT_E* code on failure; ft_last_error() then gives a
+ * human-readable reason for the calling thread.
+ *
+ * Each declaration cites the interface of the reference it replaces (paths relative to the
+ * reference checkout, npz7yyk/FlexTrain 0.1.0+e829f0c).
+ */
+#ifndef FT_ADAM_H
+#define FT_ADAM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of gradient inputs and of the low-precision parameter copy */
+enum { FT_F32 = 0, FT_F16 = 1, FT_BF16 = 2 };
+
+enum {
+    FT_OK = 0,
+    FT_EINVAL = -1,   /* bad argument (NULL, dtype code, size)                       */
+    FT_EALIGN = -2,   /* pointer not aligned to its element size                     */
+    FT_ENOENT = -3,   /* unknown optimizer id / handle                               */
+    FT_EHIP = -4,     /* a HIP runtime call failed; message carries hipGetErrorString */
+    FT_ENOMEM = -5,   /* allocation failed                                           */
+    FT_EBUSY = -6     /* handle still has work in flight                             */
+};
+
+/* Result of the gradient statistics pass (device memory, 16 bytes, 16-byte aligned). */
+typedef struct ft_grad_stats_t {
+    uint64_t nonfinite; /* number of inf/nan gradient elements                        */
+    double sumsq;       /* sum of squares of the finite unscaled gradient elements    */
+} ft_grad_stats_t;
+
+/* Per-step decision consumed by the update kernel on the device (16 bytes, 16-byte aligned). */
+typedef struct ft_step_control_t {
+    uint32_t skip;   /* non-zero: leave p, m, v and the low-precision copy untouched    */
+    float grad_mult; /* g32 = (float)g * grad_mult  (= clip_coef * 1/loss_scale)        */
+    float grad_norm; /* L2 norm of the unscaled gradient, for the caller's information  */
+    float clip_coef; /* min(1, max_norm / (norm + 1e-6)), 1 when clipping is off        */
+} ft_step_control_t;
+
+const char* ft_last_error(void);
+int ft_abi_version(void);
+
+/* Number of HIP devices visible, or a negative code. Never initialises a context beyond what
+ * hipGetDeviceCount does. */
+int ft_device_count(void);
+
+/* ---- optimizer registry ---------------------------------------------------------------
+ * Replaces create_adam / destroy_adam of the reference's pybind module
+ * (flextrain/ops/csrc/adam/cpu_adam.cpp:8-16, bodies cpu_adam_impl.cpp:143-181,297-302).
+ * The object holds the default hyper-parameters and adamw_mode; an unknown id is an error
+ * (FT_ENOENT) instead of the reference's null-pointer dereference (cpu_adam_impl.cpp:235-237).
+ */
+int ft_adam_create(int id, float lr, float beta1, float beta2, float eps, float weight_decay,
+                   int adamw_mode, int should_log);
+int ft_adam_destroy(int id);
+
+/* ---- resident update --------------------------------------------------------------------
+ * Replaces adam_update and adam_update_copy (ds_adam_step / ds_adam_step_plus_copy,
+ * flextrain/ops/csrc/adam/cpu_adam_impl.cpp:212-295; arithmetic cpu_adam.h:130-216; host
+ * scalars cpu_adam.h:67-102). Same argument order and meaning for
+ * (id, step, lr, beta1, beta2, eps, weight_decay, bias_correction, params, grads, exp_avg,
+ * exp_avg_sq[, device_params]); additions:
+ *   grad_mult   the gradient is multiplied by this fp32 factor on load (1.0f = reference)
+ *   g_dtype     gradients may be fp32 (as the reference requires), fp16 or bf16
+ *   half_out    NULL (= adam_update) or the low-precision copy (= adam_update_copy);
+ *   half_dtype  FT_F16 reproduces the reference's copy-out (simd.h:35-37); FT_BF16 writes
+ *               round-to-nearest-even bfloat16
+ *   ctl         NULL, or a device ft_step_control_t read by the kernel: it overrides
+ *               grad_mult and can turn the whole call into a no-op (skip)
+ * p, m, v: fp32, n elements, updated in place. Pointers must be aligned to their element size;
+ * full speed needs p/m/v 16-byte and 16-bit arrays 8-byte aligned at the same element offset.
+ */
+int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, float eps,
+                 float weight_decay, int bias_correction, float grad_mult, void* p, const void* g,
+                 int g_dtype, void* m, void* v, void* half_out, int half_dtype, size_t n,
+                 const void* ctl, void* stream);
+
+/* ---- gradient statistics and the skip / clip decision -----------------------------------
+ * No counterpart in the reference: it scales the loss (flextrain/engine.py:249) but never
+ * unscales, checks or clips gradients, and nothing calls DynamicLossScaler.update_scale
+ * (flextrain/loss_scaler.py:134-179). These entry points supply what that state machine needs.
+ *
+ * ft_grad_stats: one pass over g; writes (accumulate == 0) or adds (accumulate != 0) the count
+ * of inf/nan elements and the sum of squares of (float)g * pre_mult into *out (device).
+ * workspace: device scratch of at least ft_grad_stats_workspace_bytes() bytes, or NULL to use a
+ * per-device buffer the library allocates on first use (calls that share it must be ordered on
+ * one stream).
+ */
+size_t ft_grad_stats_workspace_bytes(void);
+int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate,
+                  void* workspace, size_t workspace_bytes, void* stream);
+
+/* ft_grad_control: turns statistics into the per-step decision, on the device:
+ *   skip      = stats->nonfinite != 0
+ *   norm      = sqrt(stats->sumsq)                                (double)
+ *   clip_coef = max_norm > 0 ? min(1, max_norm / (norm + 1e-6)) : 1   (double, then fp32)
+ *   grad_mult = clip_coef * inv_scale                             (one fp32 multiply)
+ */
+int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ctl_out, void* stream);
+
+/* ---- pinned host memory -------------------------------------------------------------------
+ * Replaces the pinned allocations of flextrain/memory/__init__.py:255-277 and
+ * flextrain/memory/pin_memory.py:100-171 (torch pin_memory, power-of-two rounded): exact-size,
+ * page-aligned, device-accessible host memory from hipHostMalloc. */
+int ft_pinned_alloc(size_t bytes, void** out);
+int ft_pinned_free(void* ptr);
+
+/* ---- offloaded (streamed) update --------------------------------------------------------
+ * Replaces the reference's "state lives in pinned host memory, step runs where the state is"
+ * arrangement (flextrain/optimizer.py:244-263; flextrain/memory/__init__.py:240-248,366-395:
+ * RotateContainer double buffering and the single side stream with device-wide synchronisation)
+ * by a pipeline that brings the state to the GPU in chunks: for every chunk, H2D of p/m/v
+ * (+ g when it lives on the host) on one stream, the update kernel on a second, D2H of p/m/v
+ * (+ the low-precision copy when it lives on the host) on a third, ordered per buffer slot by
+ * events, never by a device-wide wait.
+ *
+ * ft_offload_create: chunk_elems elements per chunk, n_slots (>= 2) device buffer sets.
+ * ft_offload_step:   enqueues one full step over n elements and returns; host_p/m/v are pinned
+ *                    host arrays; g and half_out are device pointers when *_on_host == 0 and
+ *                    pinned host pointers otherwise (half_out may be NULL). The step starts
+ *                    after the work already enqueued on `stream` (the producer of g and ctl),
+ *                    and `stream` is made to wait for the step's end, so later work on it sees
+ *                    the new half_out.
+ * ft_offload_wait:   blocks until the last enqueued step has finished.
+ * ft_offload_elapsed_ms: device time between the first H2D and the last D2H of the last
+ *                    finished step (valid after ft_offload_wait).
+ */
+int ft_offload_create(size_t chunk_elems, int n_slots, void** out_handle);
+int ft_offload_destroy(void* handle);
+int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, float beta2,
+                    float eps, float weight_decay, int bias_correction, float grad_mult,
+                    void* host_p, const void* g, int g_dtype, int g_on_host, void* host_m,
+                    void* host_v, void* half_out, int half_dtype, int half_on_host, size_t n,
+                    const void* ctl, void* stream);
+int ft_offload_wait(void* handle);
+int ft_offload_elapsed_ms(void* handle, float* out_ms);
+
+/* Host-link probe used to put the offloaded step next to what the link can do: copies `bytes`
+ * between pinned host and device memory `iters` times and reports GB/s (1e9 bytes/s).
+ * direction: 0 = host-to-device, 1 = device-to-host, 2 = both at once (sum of both reported).
+ * The method follows the reference's own probe (flextrain/auto_config.py:184-215). */
+int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps);
+
+/* ---- launch tuning ------------------------------------------------------------------------
+ * Grid shape of the update and statistics kernels. blocks_per_cu <= 0 restores the default.
+ * Affects speed only, never results. */
+int ft_set_launch_tuning(int adam_blocks_per_cu, int stats_blocks_per_cu);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
