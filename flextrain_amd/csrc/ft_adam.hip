@@ -16,11 +16,15 @@
 #include "ft_internal.hpp"
 #include "ft_kernels.hpp"
 
+// Launch shape of the update kernel, from sweeps on MI355X at 2e8 elements: one 64-lane wavefront
+// per workgroup, one 4-element unit per lane, one workgroup per tile, non-temporal loads and
+// stores, and at most 12 workgroups resident per compute unit. More resident wavefronts put more
+// requests in flight than HBM can serve in order and cost up to 8 % of the bandwidth.
 #ifndef FT_ADAM_BLOCK
-#define FT_ADAM_BLOCK 256
+#define FT_ADAM_BLOCK 64
 #endif
 #ifndef FT_ADAM_UNROLL
-#define FT_ADAM_UNROLL 2
+#define FT_ADAM_UNROLL 1
 #endif
 #ifndef FT_ADAM_NT_LD
 #define FT_ADAM_NT_LD true
@@ -28,8 +32,8 @@
 #ifndef FT_ADAM_NT_ST
 #define FT_ADAM_NT_ST true
 #endif
-#ifndef FT_ADAM_BLOCKS_PER_CU
-#define FT_ADAM_BLOCKS_PER_CU 8
+#ifndef FT_ADAM_WAVES_PER_CU
+#define FT_ADAM_WAVES_PER_CU 12
 #endif
 #ifndef FT_STATS_BLOCK
 #define FT_STATS_BLOCK 256
@@ -49,7 +53,8 @@ std::mutex g_mu;
 std::unordered_map<int, fth::AdamObject> g_adams;
 std::unordered_map<int, int> g_cu_count;      // device -> compute units
 std::unordered_map<int, void*> g_stats_ws;    // device -> library-owned statistics scratch
-int g_adam_blocks_per_cu = FT_ADAM_BLOCKS_PER_CU;
+int g_adam_waves_per_cu = FT_ADAM_WAVES_PER_CU;
+std::unordered_map<int, int> g_lds_per_cu;   // device -> bytes of LDS per compute unit
 int g_stats_blocks_per_cu = FT_STATS_BLOCKS_PER_CU;
 
 constexpr int kMaxStatsBlocks = 8192;
@@ -93,6 +98,30 @@ int cu_count()
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
     g_cu_count[dev] = n;
     return n;
+}
+
+// Dynamic LDS requested per workgroup of the update kernel. The kernel never touches it: the
+// allocation only bounds how many workgroups fit on a compute unit at once.
+unsigned adam_throttle_lds_bytes()
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 0;
+    std::lock_guard<std::mutex> lk(g_mu);
+    const int waves = g_adam_waves_per_cu;
+    constexpr int kMaxResident = 32 * 64 / FT_ADAM_BLOCK;  // hardware limit: 32 wavefronts per CU
+    if (waves >= kMaxResident) return 0;
+    auto it = g_lds_per_cu.find(dev);
+    int lds = 0;
+    if (it != g_lds_per_cu.end()) {
+        lds = it->second;
+    } else {
+        if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || lds <= 0)
+            lds = 160 * 1024;
+        g_lds_per_cu[dev] = lds;
+    }
+    int per_wg = (lds / waves) / 512 * 512;
+    if (per_wg > 64 * 1024) per_wg = 64 * 1024;
+    return static_cast<unsigned>(per_wg);
 }
 
 ftk::AdamConsts make_consts(uint64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -180,12 +209,12 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.n = nvec;
         a.c = c;
         constexpr size_t kTile = static_cast<size_t>(FT_ADAM_BLOCK) * FT_ADAM_UNROLL;
-        size_t blocks = (nvec + kTile - 1) / kTile;
-        const size_t cap = static_cast<size_t>(cu_count()) * static_cast<size_t>(g_adam_blocks_per_cu);
+        size_t blocks = (nvec + kTile - 1) / kTile;  // one tile per workgroup ...
+        const size_t cap = 0x7fffffffu;              // ... unless the grid would overflow
         if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL(
             (ftk::adam_vec_kernel<GT, HT, FT_ADAM_BLOCK, FT_ADAM_UNROLL, FT_ADAM_NT_LD, FT_ADAM_NT_ST>),
-            dim3(static_cast<unsigned>(blocks)), dim3(FT_ADAM_BLOCK), 0, stream, a);
+            dim3(static_cast<unsigned>(blocks)), dim3(FT_ADAM_BLOCK), adam_throttle_lds_bytes(), stream, a);
         FT_HIP(hipGetLastError());
     }
     int rc = scalar_part(0, head);
@@ -381,10 +410,10 @@ int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ct
     return FT_OK;
 }
 
-int ft_set_launch_tuning(int adam_blocks_per_cu, int stats_blocks_per_cu)
+int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu)
 {
     std::lock_guard<std::mutex> lk(g_mu);
-    g_adam_blocks_per_cu = adam_blocks_per_cu > 0 ? adam_blocks_per_cu : FT_ADAM_BLOCKS_PER_CU;
+    g_adam_waves_per_cu = adam_waves_per_cu > 0 ? adam_waves_per_cu : FT_ADAM_WAVES_PER_CU;
     g_stats_blocks_per_cu = stats_blocks_per_cu > 0 ? stats_blocks_per_cu : FT_STATS_BLOCKS_PER_CU;
     return FT_OK;
 }

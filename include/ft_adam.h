@@ -154,9 +154,11 @@ int ft_offload_elapsed_ms(void* handle, float* out_ms);
 int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps);
 
 /* ---- launch tuning ------------------------------------------------------------------------
- * Grid shape of the update and statistics kernels. blocks_per_cu <= 0 restores the default.
- * Affects speed only, never results. */
-int ft_set_launch_tuning(int adam_blocks_per_cu, int stats_blocks_per_cu);
+ * adam_waves_per_cu: how many 64-lane workgroups of the update kernel may be resident on one
+ * compute unit (an occupancy throttle; 32 or more = no throttle). stats_blocks_per_cu: grid size
+ * of the statistics kernel in 256-thread blocks per compute unit. A value <= 0 restores the
+ * default. Affects speed only, never results. */
+int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu);
 
 #ifdef __cplusplus
 }

@@ -73,3 +73,34 @@ def to_np(t: torch.Tensor) -> np.ndarray:
 def half_bits(t: torch.Tensor) -> np.ndarray:
     """uint16 bit patterns of an fp16/bf16 tensor."""
     return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def max_ulp_gpu(dev: torch.Tensor, host: np.ndarray, chunk: int = 1 << 26) -> int:
+    """Largest ULP distance between a GPU tensor (fp32, or fp16/bf16) and host data of the same
+    format (float32 array, or uint16 bit patterns), evaluated on the GPU chunk by chunk. NaN
+    against NaN counts as equal, NaN against a number as a huge distance."""
+    n = dev.numel()
+    assert host.shape[0] == n
+    if dev.dtype == torch.float32:
+        width, idt, exp_mask, view = 32, torch.int32, 0x7f800000, np.int32
+    elif dev.dtype == torch.float16:
+        width, idt, exp_mask, view = 16, torch.int16, 0x7c00, np.int16
+    elif dev.dtype == torch.bfloat16:
+        width, idt, exp_mask, view = 16, torch.int16, 0x7f80, np.int16
+    else:
+        raise TypeError(dev.dtype)
+    mag = (1 << (width - 1)) - 1
+    worst = 0
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        a = dev[lo:hi].view(idt).to(torch.int64)
+        b = torch.from_numpy(host[lo:hi].view(view)).to(dev.device).to(torch.int64)
+        a_mag, b_mag = a & mag, b & mag
+        a_nan, b_nan = a_mag > exp_mask, b_mag > exp_mask
+        oa = torch.where(a < 0, -a_mag, a_mag)
+        ob = torch.where(b < 0, -b_mag, b_mag)
+        d = (oa - ob).abs()
+        d = torch.where(a_nan & b_nan, torch.zeros_like(d), d)
+        d = torch.where(a_nan ^ b_nan, torch.full_like(d, 1 << 40), d)
+        worst = max(worst, int(d.max().item()))
+    return worst
