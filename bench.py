@@ -28,7 +28,7 @@ N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 8
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
 # profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": None, "cfg3": None, "cfg4": None}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_727_000, "cfg3": None, "cfg4": None}
 
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
 
@@ -108,6 +108,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="before the timed region, run 3 plain device copies of one fp32 array of the workload "
+                         "(known size: 4 bytes/element read + 4 written) so that a rocprofv3 --pmc run of this "
+                         "command holds a reference dispatch to scale FETCH_SIZE / WRITE_SIZE with")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the optimizer step of ONE GPU's partition; --gpus must be 1 "
@@ -152,6 +156,13 @@ def main() -> int:
             eng._step(group, h, p, g, m, v, control=ctl)
         else:
             eng._step(group, h, p, g, m, v)
+
+    if args.calibration_copy:
+        scratch = torch.empty_like(p)
+        for _ in range(3):
+            scratch.copy_(p)
+        torch.cuda.synchronize()
+        del scratch
 
     for _ in range(args.warmup):
         one_step()
