@@ -73,14 +73,17 @@ class FlexTrainCPUOptimizer(ABC):
             )
 
     def _allocate(self, numel: int, dtype: torch.dtype, fill: str) -> Tensor:
-        """A flat buffer on ``state_device`` (pinned when that is the host)."""
+        """A flat buffer on ``state_device`` (pinned, exact size, when that is the host)."""
         if self.state_device == "cpu":
-            make = {"zeros": torch.zeros, "empty": torch.empty, "randn": torch.randn}[fill]
-            t = make(numel, dtype=dtype)
-            return t.pin_memory() if numel > 0 else t
-        device = torch.device("cuda", torch.cuda.current_device())
-        make = {"zeros": torch.zeros, "empty": torch.empty, "randn": torch.randn}[fill]
-        return make(numel, dtype=dtype, device=device)
+            from .memory import pinned_empty
+            t = pinned_empty(numel, dtype)
+        else:
+            t = torch.empty(numel, dtype=dtype, device=torch.device("cuda", torch.cuda.current_device()))
+        if fill == "zeros":
+            t.zero_()
+        elif fill == "randn":
+            t.normal_()
+        return t
 
     @torch.no_grad()
     def profile_step(self, numel: int, device_dtype: torch.dtype, master_dtype: torch.dtype):
@@ -206,8 +209,8 @@ class FlexTrainOptimizer:
         # fp32 master copy: resident (aliases the device buffer when that is fp32 already) or
         # pinned host memory when offloaded.
         if self._offload:
-            self._master_para = torch.zeros(total_numel, dtype=master_dtype).pin_memory() \
-                if total_numel else torch.zeros(0, dtype=master_dtype)
+            from .memory import pinned_empty
+            self._master_para = pinned_empty(total_numel, master_dtype)
             self._master_para.copy_(self._device_para)
         elif device_dtype == master_dtype:
             self._master_para = self._device_para

@@ -1,0 +1,174 @@
+"""GPU tests of the pinned-host <-> HBM pipeline: the streamed step must give the bits of the
+resident step (and so of the oracle), whatever the chunking, slot count, or where gradients and
+the low-precision copy live."""
+import numpy as np
+import pytest
+import torch
+
+from _util import CODE, F16, HALF_ULP, MASTER_ULP, half_bits, max_ulp, to_np
+
+pytestmark = pytest.mark.gpu
+
+HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
+
+
+def _host_state(n, seed):
+    from flextrain_amd.memory import pinned_empty
+    rng = np.random.default_rng(seed)
+    p, m, v = (pinned_empty(n, torch.float32) for _ in range(3))
+    p.copy_(torch.from_numpy(rng.normal(0, 0.02, n).astype(np.float32)))
+    m.copy_(torch.from_numpy(rng.normal(0, 1e-4, n).astype(np.float32)))
+    v.copy_(torch.from_numpy(rng.uniform(0, 1e-6, n).astype(np.float32)))
+    return p, m, v
+
+
+def _oracle(oracle, p, g, m, v, step, half_dtype, grad_mult=1.0):
+    pn, mn, vn = p.numpy().copy(), m.numpy().copy(), v.numpy().copy()
+    gn = to_np(g)
+    if g.dtype == torch.float16:
+        gn = gn.view(np.uint16)
+    hn = np.zeros(pn.shape[0], np.uint16) if half_dtype is not None else None
+    oracle.adam_step(pn, gn, mn, vn, step=step, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
+                     weight_decay=HP["weight_decay"], g_dtype=CODE[g.dtype], grad_mult=grad_mult, half_out=hn,
+                     half_dtype=CODE[half_dtype] if half_dtype is not None else F16)
+    return pn, mn, vn, hn
+
+
+def _assert_equal_bits(tag, p, m, v, h, want, half_dtype):
+    pn, mn, vn, hn = want
+    worst = dict(p=max_ulp(p.numpy(), pn), m=max_ulp(m.numpy(), mn), v=max_ulp(v.numpy(), vn))
+    if h is not None:
+        hb = half_bits(h)
+        worst["h"] = max_ulp(hb, hn, bf16=True) if half_dtype == torch.bfloat16 else max_ulp(hb.view(np.float16), hn.view(np.float16))
+    print(f"[{tag}] worst ULP distance: {worst}", flush=True)
+    assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst.get("h", 0) <= HALF_ULP, (tag, worst)
+
+
+def test_pinned_allocations(cuda):
+    from flextrain_amd.memory import allocate_memory, allocate_memory_chunks, allocate_pin_memory_blocks, pinned_empty
+    t = pinned_empty(1_000_003, torch.float32)
+    assert t.is_pinned() and t.numel() == 1_000_003 and t.data_ptr() % 4096 == 0
+    z = allocate_memory(12345, torch.float32, "cpu")
+    assert z.is_pinned() and not z.any()
+    blocks = allocate_pin_memory_blocks(1000, torch.float16, (2, 3))
+    assert len(blocks) == 2 and len(blocks[0]) == 3
+    flat = [b for row in blocks for b in row]
+    assert all(b.is_pinned() and b.numel() == 1000 and b.dtype == torch.float16 and not b.any() for b in flat)
+    assert all(b.data_ptr() % 4096 == 0 for b in flat)
+    spans = sorted((b.data_ptr(), b.data_ptr() + 2000) for b in flat)
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))  # disjoint
+    nested = allocate_memory_chunks(64, (2, 2), torch.float32, "cpu")
+    assert nested[1][1].is_pinned()
+    dev = allocate_memory_chunks(64, 3, torch.float32, cuda)
+    assert dev.shape == (3, 64) and dev.is_cuda
+    empty = allocate_pin_memory_blocks(0, torch.float32, 2)
+    assert len(empty) == 2 and empty[0].numel() == 0
+    # round trip through the GPU
+    t.copy_(torch.arange(1_000_003, dtype=torch.float32))
+    d = t.to(cuda, non_blocking=True)
+    torch.cuda.synchronize()
+    assert d[-1].item() == 1_000_002.0
+
+
+def test_data_stream_orders_copies_behind_their_producer(cuda):
+    from flextrain_amd.memory import FlexTrainDataStream, pinned_empty
+    ds = FlexTrainDataStream()
+    n = 8_000_000
+    src = torch.zeros(n, device=cuda)
+    dst = pinned_empty(n, torch.float32)
+    dst.zero_()
+    ran = []
+    for i in range(3):
+        src.add_(1.0)  # producer on the current stream
+        ds.submit(lambda: dst.copy_(src, non_blocking=True))
+        ds.submit(lambda: ran.append(i), stream_execution=False)
+        handle = ds.execute()
+        ds.wait()  # the producer of the next round must not overwrite src before the copy has read it
+        handle.wait()
+        assert dst[0].item() == float(i + 1) and dst[-1].item() == float(i + 1)
+    assert ran == [0, 1, 2] and ds.is_empty()
+    ds.synchronize()
+
+
+@pytest.mark.parametrize("slots", [2, 3])
+@pytest.mark.parametrize("n,chunk", [(1_000_003, 1 << 16), (300_000, 1 << 20), (4 * (1 << 16), 1 << 16)])
+def test_streamed_step_device_grads(cuda, oracle, n, chunk, slots):
+    """Master state in pinned host memory, bf16 grads and bf16 copy on the GPU (the offloaded
+    configuration), several chunks, ragged last chunk, two steps in a row."""
+    from flextrain_amd import FlexTrainCPUAdam
+    eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=slots, **HP)
+    p, m, v = _host_state(n, seed=n)
+    h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    gen = torch.Generator(device=cuda).manual_seed(1)
+    for t in (1, 2):
+        g = (torch.randn(n, device=cuda, generator=gen) * 1e-3).to(torch.bfloat16)
+        want = _oracle(oracle, p, g, m, v, t, torch.bfloat16)
+        eng._step({"step": t}, h, p, g, m, v)
+        _assert_equal_bits(f"offload n={n} chunk={chunk} slots={slots} t={t}", p, m, v, h, want, torch.bfloat16)
+
+
+def test_streamed_step_reference_layout(cuda, oracle):
+    """Everything in pinned host memory with fp32 gradients and an fp16 copy: the layout the
+    reference's coordinator hands to the step."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.memory import pinned_empty
+    n = 700_001
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 17, offload_slots=2, **HP)
+    p, m, v = _host_state(n, seed=3)
+    g = pinned_empty(n, torch.float32)
+    g.copy_(torch.randn(n) * 1e-3)
+    h = pinned_empty(n, torch.float16)
+    h.zero_()
+    want = _oracle(oracle, p, g, m, v, 9, torch.float16)
+    eng._step({"step": 9}, h, p, g, m, v)
+    _assert_equal_bits("host layout", p, m, v, h, want, torch.float16)
+    assert eng.last_offload_ms() > 0
+
+
+def test_streamed_equals_resident_bit_for_bit(cuda):
+    from flextrain_amd import FlexTrainCPUAdam
+    n = 3_000_017
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 18, offload_slots=3, **HP)
+    p, m, v = _host_state(n, seed=8)
+    g = (torch.randn(n, device=cuda) * 1e-3 * 512).to(torch.float16)
+    dp, dm, dv = p.to(cuda), m.to(cuda), v.to(cuda)
+    dh = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    for t in range(1, 4):
+        eng._step({"step": t}, dh, dp, g, dm, dv, grad_mult=1.0 / 512)
+        eng._step({"step": t}, h, p, g, m, v, grad_mult=1.0 / 512)
+    torch.cuda.synchronize()
+    assert torch.equal(dp.cpu(), p) and torch.equal(dm.cpu(), m) and torch.equal(dv.cpu(), v) and torch.equal(dh, h)
+
+
+def test_non_blocking_step_and_explicit_wait(cuda, oracle):
+    from flextrain_amd import FlexTrainCPUAdam
+    n = 2_000_000
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 18, **HP)
+    p, m, v = _host_state(n, seed=5)
+    g = (torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16)
+    want = _oracle(oracle, p, g, m, v, 1, None)
+    eng._step({"step": 1}, None, p, g, m, v, blocking=False)
+    eng.synchronize()
+    _assert_equal_bits("non-blocking", p, m, v, None, want, None)
+
+
+def test_pageable_host_memory_is_refused(cuda):
+    from flextrain_amd import FlexTrainCPUAdam
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 16, **HP)
+    n = 1000
+    p, m, v = (torch.zeros(n) for _ in range(3))
+    g = torch.zeros(n, device=cuda)
+    with pytest.raises(ValueError, match="pinned"):
+        eng._step({"step": 1}, None, p, g, m, v)
+
+
+def test_link_probe_reports_sane_numbers(cuda):
+    import ctypes
+    from flextrain_amd import _C
+    lib = _C.lib()
+    out = ctypes.c_double()
+    for direction in (0, 1, 2):
+        _C.check("ft_link_bandwidth", lib.ft_link_bandwidth(256 << 20, 4, direction, ctypes.byref(out)))
+        print(f"[link] direction {direction}: {out.value:.1f} GB/s", flush=True)
+        assert 1.0 < out.value < 1000.0
