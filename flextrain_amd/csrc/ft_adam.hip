@@ -18,7 +18,7 @@
 
 // Launch shape of the update kernel, from sweeps on MI355X at 2e8 elements: one 64-lane wavefront
 // per workgroup, one 4-element unit per lane, one workgroup per tile, non-temporal loads and
-// stores, and at most 12 workgroups resident per compute unit. More resident wavefronts put more
+// stores, and at most 11 workgroups resident per compute unit. More resident wavefronts put more
 // requests in flight than HBM can serve in order and cost up to 8 % of the bandwidth.
 #ifndef FT_ADAM_BLOCK
 #define FT_ADAM_BLOCK 64
@@ -33,7 +33,7 @@
 #define FT_ADAM_NT_ST true
 #endif
 #ifndef FT_ADAM_WAVES_PER_CU
-#define FT_ADAM_WAVES_PER_CU 12
+#define FT_ADAM_WAVES_PER_CU 11
 #endif
 #ifndef FT_STATS_BLOCK
 #define FT_STATS_BLOCK 256
@@ -42,7 +42,7 @@
 #define FT_STATS_UNROLL 4
 #endif
 #ifndef FT_STATS_BLOCKS_PER_CU
-#define FT_STATS_BLOCKS_PER_CU 8
+#define FT_STATS_BLOCKS_PER_CU 4
 #endif
 
 namespace {
