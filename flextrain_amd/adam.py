@@ -116,6 +116,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
         grad_mult: float = 1.0,
         control: Optional[Tensor] = None,
         blocking: Optional[bool] = None,
+        guard_stream: bool = True,
     ):
         """One Adam/AdamW update of a contiguous segment, in place.
 
@@ -126,7 +127,11 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
         Resident mode (``full_parameter`` on the GPU): the kernel is enqueued on torch's current
         stream and the call returns at once. Offloaded mode (``full_parameter`` in pinned host
         memory): the chunk pipeline is enqueued; with ``blocking`` (default in this mode) the call
-        returns when the host arrays hold the new values, as the reference's host step does.
+        returns when the host arrays hold the new values, as the reference's host step does. With
+        ``blocking=False`` the call returns at once; torch's current stream is then made to wait
+        for the step's kernels (so that the gradients may be overwritten and the new copy read)
+        unless ``guard_stream=False``, in which case the caller orders its own work with
+        ``stream_wait()`` / ``synchronize()``.
         """
         assert STEP_KEY in group_args, f"Key '{STEP_KEY}' not found in parameter group arguments."
         self._set_defaults_args(group_args)
@@ -184,11 +189,21 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             _C.current_stream_ptr()))
         if blocking is None or blocking:
             _C.check("ft_offload_wait", self._lib.ft_offload_wait(engine))
+        elif guard_stream and (gradient.is_cuda or (half_parameter is not None and half_parameter.is_cuda)):
+            # later work on the caller's stream may overwrite the gradients or read the new copy
+            _C.check("ft_offload_stream_wait", self._lib.ft_offload_stream_wait(engine, _C.current_stream_ptr(), 0))
 
     def synchronize(self):
-        """Waits for the last offloaded step (no-op if none was enqueued)."""
+        """Waits for every offloaded step enqueued so far (no-op if none was)."""
         if self._engine is not None:
             _C.check("ft_offload_wait", self._lib.ft_offload_wait(self._engine))
+
+    def stream_wait(self, write_back: bool = False):
+        """Makes torch's current stream wait for the last offloaded step: for its kernels, or with
+        ``write_back`` for its copies back to host memory."""
+        if self._engine is not None:
+            _C.check("ft_offload_stream_wait", self._lib.ft_offload_stream_wait(
+                self._engine, _C.current_stream_ptr(), 1 if write_back else 0))
 
     def last_offload_ms(self) -> float:
         """Device time of the last finished offloaded step, first H2D to last D2H."""

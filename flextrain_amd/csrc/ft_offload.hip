@@ -9,6 +9,7 @@
 #include <string.h>
 
 #include <chrono>
+#include <deque>
 #include <vector>
 
 #include "ft_internal.hpp"
@@ -25,6 +26,22 @@ struct Slot {
     bool used = false;
 };
 
+// Host memory a step writes back to, and the event that marks its last D2H.
+struct Pending {
+    uintptr_t lo[4], hi[4];
+    int ranges = 0;
+    hipEvent_t done = nullptr;
+    bool overlaps(const Pending& o) const
+    {
+        for (int i = 0; i < ranges; ++i)
+            for (int j = 0; j < o.ranges; ++j)
+                if (lo[i] < o.hi[j] && o.lo[j] < hi[i]) return true;
+        return false;
+    }
+};
+
+constexpr size_t kMaxPending = 8;
+
 struct Engine {
     uint32_t magic = 0x46544f45;  // "FTOE"
     int device = 0;
@@ -36,6 +53,8 @@ struct Engine {
     hipEvent_t ev_end = nullptr;    // last D2H of the last step
     hipEvent_t ev_kernels = nullptr;  // last kernel of the last step
     bool stepped = false;
+    std::deque<Pending> recent;        // steps whose write-back may still be in flight, oldest first
+    std::vector<hipEvent_t> free_events;
 };
 
 Engine* as_engine(void* h)
@@ -77,6 +96,9 @@ void destroy_engine(Engine* e)
     if (e->ev_begin) (void)hipEventDestroy(e->ev_begin);
     if (e->ev_end) (void)hipEventDestroy(e->ev_end);
     if (e->ev_kernels) (void)hipEventDestroy(e->ev_kernels);
+    for (Pending& pd : e->recent)
+        if (pd.done) (void)hipEventDestroy(pd.done);
+    for (hipEvent_t ev : e->free_events) (void)hipEventDestroy(ev);
     e->magic = 0;
     delete e;
 }
@@ -133,6 +155,11 @@ int ft_offload_create(size_t chunk_elems, int n_slots, void** out_handle)
     if ((err = hipEventCreate(&e->ev_begin)) != hipSuccess) return bail(err, "hipEventCreate");
     if ((err = hipEventCreate(&e->ev_end)) != hipSuccess) return bail(err, "hipEventCreate");
     if ((err = hipEventCreate(&e->ev_kernels)) != hipSuccess) return bail(err, "hipEventCreate");
+    for (size_t i = 0; i < kMaxPending; ++i) {
+        hipEvent_t ev = nullptr;
+        if ((err = hipEventCreateWithFlags(&ev, hipEventDisableTiming)) != hipSuccess) return bail(err, "hipEventCreate");
+        e->free_events.push_back(ev);
+    }
     for (Slot& s : e->slots) {
         if ((err = hipMalloc(reinterpret_cast<void**>(&s.p), chunk_elems * 4)) != hipSuccess) return bail(err, "hipMalloc");
         if ((err = hipMalloc(reinterpret_cast<void**>(&s.m), chunk_elems * 4)) != hipSuccess) return bail(err, "hipMalloc");
@@ -191,12 +218,32 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
         fth::make_consts(step, lr, beta1, beta2, eps, weight_decay, bias_correction != 0, o.adamw_mode, grad_mult);
     hipStream_t user = static_cast<hipStream_t>(stream);
 
-    // The pipeline starts after the producer of g/ctl, and after the previous step's last D2H
-    // (a chunk's host copy must be complete before the next step reads it again).
+    // Host ranges this step writes back to. A later step that touches any of them must not start
+    // reading before this step's last D2H; steps on disjoint memory (other units, other parameter
+    // groups) are free to overlap with it.
+    Pending mine;
+    auto add_range = [&](const void* ptr, size_t bytes) {
+        mine.lo[mine.ranges] = reinterpret_cast<uintptr_t>(ptr);
+        mine.hi[mine.ranges] = reinterpret_cast<uintptr_t>(ptr) + bytes;
+        ++mine.ranges;
+    };
+    add_range(host_p, n * 4);
+    add_range(host_m, n * 4);
+    add_range(host_v, n * 4);
+    if (half_out && half_on_host) add_range(half_out, n * 2);
+
+    // The pipeline starts after the producer of g/ctl on the caller's stream ...
     FT_HIP(hipEventRecord(e->ev_user, user));
     FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_user, 0));
     FT_HIP(hipStreamWaitEvent(e->s_k, e->ev_user, 0));
-    if (e->stepped) FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_end, 0));
+    // ... and after the newest earlier step that wrote to the same host memory (the D2H stream is
+    // in order, so that one event covers all older ones).
+    for (auto it = e->recent.rbegin(); it != e->recent.rend(); ++it) {
+        if (it->overlaps(mine)) {
+            FT_HIP(hipStreamWaitEvent(e->s_h2d, it->done, 0));
+            break;
+        }
+    }
     FT_HIP(hipEventRecord(e->ev_begin, e->s_h2d));
 
     float* hp = static_cast<float*>(host_p);
@@ -238,10 +285,29 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     FT_HIP(hipEventRecord(e->ev_kernels, e->s_k));
     FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
     e->stepped = true;
-    // Later work on the producer stream sees the new device-resident low-precision copy (kernels)
-    // and may reuse g (also kernels); waiting for the last D2H as well keeps "step finished" simple.
-    FT_HIP(hipStreamWaitEvent(user, e->ev_kernels, 0));
-    FT_HIP(hipStreamWaitEvent(user, e->ev_end, 0));
+
+    // Remember this step's write-back. When the list is full the oldest entry is retired; every
+    // later H2D is then ordered behind it, which costs nothing once it has long finished.
+    if (e->free_events.empty()) {
+        Pending& old = e->recent.front();
+        FT_HIP(hipStreamWaitEvent(e->s_h2d, old.done, 0));
+        e->free_events.push_back(old.done);
+        e->recent.pop_front();
+    }
+    mine.done = e->free_events.back();
+    e->free_events.pop_back();
+    FT_HIP(hipEventRecord(mine.done, e->s_d2h));
+    e->recent.push_back(mine);
+    return FT_OK;
+}
+
+int ft_offload_stream_wait(void* handle, void* stream, int what)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    if (what != 0 && what != 1) return fth::fail(FT_EINVAL, "what must be 0 (kernels) or 1 (write-back)");
+    if (!e->stepped) return FT_OK;
+    FT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), what == 0 ? e->ev_kernels : e->ev_end, 0));
     return FT_OK;
 }
 
@@ -252,6 +318,9 @@ int ft_offload_wait(void* handle)
     if (!e->stepped) return FT_OK;
     FT_HIP(hipEventSynchronize(e->ev_end));
     FT_HIP(hipEventSynchronize(e->ev_kernels));
+    // everything enqueued so far has finished: nothing is pending any more
+    for (Pending& pd : e->recent) e->free_events.push_back(pd.done);
+    e->recent.clear();
     return FT_OK;
 }
 

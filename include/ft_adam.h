@@ -130,12 +130,15 @@ int ft_pinned_free(void* ptr);
  * ft_offload_step:   enqueues one full step over n elements and returns; host_p/m/v are pinned
  *                    host arrays; g and half_out are device pointers when *_on_host == 0 and
  *                    pinned host pointers otherwise (half_out may be NULL). The step starts
- *                    after the work already enqueued on `stream` (the producer of g and ctl),
- *                    and `stream` is made to wait for the step's end, so later work on it sees
- *                    the new half_out.
- * ft_offload_wait:   blocks until the last enqueued step has finished.
+ *                    after the work already enqueued on `stream` (the producer of g and ctl).
+ *                    Steps on the same host memory run in the order they were enqueued; steps on
+ *                    disjoint host memory (other units, other parameter groups) overlap.
+ * ft_offload_stream_wait: makes `stream` wait, on the device, for the last enqueued step:
+ *                    what == 0 for its kernels (g may then be overwritten and a device-resident
+ *                    half_out read), what == 1 for its write-back to host memory.
+ * ft_offload_wait:   blocks the calling thread until everything enqueued so far has finished.
  * ft_offload_elapsed_ms: device time between the first H2D and the last D2H of the last
- *                    finished step (valid after ft_offload_wait).
+ *                    enqueued step (waits for it).
  */
 int ft_offload_create(size_t chunk_elems, int n_slots, void** out_handle);
 int ft_offload_destroy(void* handle);
@@ -144,6 +147,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
                     void* host_p, const void* g, int g_dtype, int g_on_host, void* host_m,
                     void* host_v, void* half_out, int half_dtype, int half_on_host, size_t n,
                     const void* ctl, void* stream);
+int ft_offload_stream_wait(void* handle, void* stream, int what);
 int ft_offload_wait(void* handle);
 int ft_offload_elapsed_ms(void* handle, float* out_ms);
 

@@ -172,3 +172,96 @@ def test_link_probe_reports_sane_numbers(cuda):
         _C.check("ft_link_bandwidth", lib.ft_link_bandwidth(256 << 20, 4, direction, ctypes.byref(out)))
         print(f"[link] direction {direction}: {out.value:.1f} GB/s", flush=True)
         assert 1.0 < out.value < 1000.0
+
+
+def test_steps_on_disjoint_memory_overlap_and_same_memory_stay_ordered(cuda, oracle):
+    """Per-unit use: many non-blocking steps in a row, each on its own host arrays, then two on the
+    same arrays; every result must equal the oracle's, and more steps than the engine tracks
+    individually (8) must still be ordered correctly."""
+    from flextrain_amd import FlexTrainCPUAdam
+    n, units = 400_000, 12
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 17, offload_slots=2, **HP)
+    state = [_host_state(n, seed=50 + u) for u in range(units)]
+    grads = [(torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16) for _ in range(units)]
+    halves = [torch.zeros(n, dtype=torch.bfloat16, device=cuda) for _ in range(units)]
+    want = [_oracle(oracle, *(state[u][0], grads[u], state[u][1], state[u][2]), 3, torch.bfloat16) for u in range(units)]
+    for u in range(units):
+        p, m, v = state[u]
+        eng._step({"step": 3}, halves[u], p, grads[u], m, v, blocking=False, guard_stream=False)
+    # unit 0 again, twice, on the same memory: must see the result of the earlier step
+    p, m, v = state[0]
+    pn, mn, vn, _ = want[0]
+    for t in (4, 5):
+        eng._step({"step": t}, halves[0], p, grads[0], m, v, blocking=False, guard_stream=False)
+        hn = np.zeros(n, np.uint16)
+        oracle.adam_step(pn, to_np(grads[0]), mn, vn, step=t, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
+                         weight_decay=HP["weight_decay"], g_dtype=CODE[torch.bfloat16], half_out=hn, half_dtype=CODE[torch.bfloat16])
+    want[0] = (pn, mn, vn, hn)
+    eng.stream_wait()
+    eng.synchronize()
+    for u in range(units):
+        p, m, v = state[u]
+        _assert_equal_bits(f"unit {u}", p, m, v, halves[u], want[u], torch.bfloat16)
+
+
+def test_config5_offloaded_7b_optimizer(cuda, oracle):
+    """The offloaded Llama-7B optimizer at the largest size this machine can pin (all 32 layers +
+    embedding + lm_head = 6.74e9 elements need 81 GB of pinned memory; a machine that refuses that
+    much runs the largest whole-layer prefix): 64 Mi-element chunks, one AdamW step at t = 100.
+    Checked by (1) the oracle on three whole chunks (first, middle, last ragged one) and
+    (2) bit-equality with the resident kernel on every chunk."""
+    import gc
+    from flextrain_amd import FlexTrainCPUAdam, _C
+    from flextrain_amd.memory import pinned_empty
+    layer, chunk = 202_383_360, 64 * 1024 * 1024
+    layers, state = 32, None
+    while state is None:
+        n = layers * layer + 2 * 4096 * 32000
+        try:
+            state = tuple(pinned_empty(n, torch.float32) for _ in range(3))
+            del_me = pinned_empty(1 << 30, torch.uint8)
+            del del_me
+        except _C.FtError:
+            state = None
+            gc.collect()
+            layers -= 1
+            assert layers >= 1
+    p, m, v = state
+    print(f"[cfg5] pinned {3 * n * 4 / 1e9:.1f} GB: {layers} of 32 layers, {n} elements, {-(-n // chunk)} chunks", flush=True)
+    g = torch.empty(n, dtype=torch.bfloat16, device=cuda)
+    h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    gen = torch.Generator(device=cuda).manual_seed(0)
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        p[lo:hi].copy_(torch.randn(hi - lo, device=cuda, generator=gen) * 0.02)
+        m[lo:hi].copy_(torch.randn(hi - lo, device=cuda, generator=gen) * 1e-4)
+        v[lo:hi].copy_(torch.rand(hi - lo, device=cuda, generator=gen) * 1e-6)
+        g[lo:hi] = (torch.randn(hi - lo, device=cuda, generator=gen) * 1e-3).to(torch.bfloat16)
+    torch.cuda.synchronize()
+    nchunks = -(-n // chunk)
+    probes = sorted({0, nchunks // 2, nchunks - 1})
+    want = {}
+    for c in probes:
+        lo, hi = c * chunk, min(n, (c + 1) * chunk)
+        want[c] = _oracle(oracle, p[lo:hi], g[lo:hi], m[lo:hi], v[lo:hi], 100, torch.bfloat16)
+    # resident results for every chunk, kept as 64-bit checksums of the raw bits
+    res = FlexTrainCPUAdam(**HP)
+    sums = []
+    for lo in range(0, n, chunk):
+        hi = min(n, lo + chunk)
+        dp, dm, dv = p[lo:hi].to(cuda), m[lo:hi].to(cuda), v[lo:hi].to(cuda)
+        dh = torch.empty(hi - lo, dtype=torch.bfloat16, device=cuda)
+        res._step({"step": 100}, dh, dp, g[lo:hi], dm, dv)
+        sums.append(tuple(int(t.view(torch.int32).to(torch.int64).sum().item()) for t in (dp, dm, dv)) +
+                    (int(dh.view(torch.int16).to(torch.int64).sum().item()),))
+    eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=3, **HP)
+    eng._step({"step": 100}, h, p, g, m, v)
+    print(f"[cfg5] streamed step: {eng.last_offload_ms():.1f} ms, {n * 12 / eng.last_offload_ms() / 1e6:.1f} GB/s each way", flush=True)
+    for c in probes:
+        lo, hi = c * chunk, min(n, (c + 1) * chunk)
+        _assert_equal_bits(f"cfg5 chunk {c}", p[lo:hi], m[lo:hi], v[lo:hi], h[lo:hi], want[c], torch.bfloat16)
+    for i, lo in enumerate(range(0, n, chunk)):
+        hi = min(n, lo + chunk)
+        got = tuple(int(t[lo:hi].to(cuda).view(torch.int32).to(torch.int64).sum().item()) for t in (p, m, v)) + \
+            (int(h[lo:hi].view(torch.int16).to(torch.int64).sum().item()),)
+        assert got == sums[i], f"chunk {i}: streamed and resident results differ"
