@@ -1,0 +1,206 @@
+"""Per-unit optimizer pipeline: the caller of the step, re-expressed for a GPU optimizer.
+
+Mirror of the optimizer-step part of the reference's ``FlexTrainOptsCoordinator``
+(``flextrain/memory/coordinator/optimizer.py``): the hooks a training loop calls around each
+unit's backward pass (``pre_unit_backward``, ``post_micro_batch_backward``,
+``clear_backward_pipeline``, ``:771-817,855-888``), buffer rotation (``:494-498``), planning a
+unit's step contexts (``:605-682``) and executing one micro-batch's share of them (``:684-696``).
+
+What is kept: the schedule. While unit ``u`` runs backward, the optimizer steps unit ``u+1``
+whose gradients are complete, one equal share per micro-batch, so the update is spread between
+the backward kernels instead of arriving as one burst. Master parameters and Adam states of every
+unit live in pinned host memory as ``[master | exp_avg | exp_avg_sq]`` blocks (``:201-210``) --
+or in HBM when ``offload=False`` -- and are seeded from the units' low-precision parameters
+(``:239-350``).
+
+What changes because the optimizer runs on the GPU:
+  * gradients never leave the GPU: there is no reduce-scatter + converting D2H hop
+    (``:534-583``), so the step of a unit follows its backward by one unit, not two;
+  * the master state of the unit being stepped streams H2D / D2H through the offload engine,
+    share by share, overlapping with the next unit's backward; ordering is by events on the
+    buffers involved, never by a device-wide synchronisation (``:819-823``);
+  * the updated low-precision parameters are written by the update kernel straight into the
+    unit's parameter buffer in HBM: no H2D copy of new parameters afterwards.
+Left out (other subsystems): the forward/backward alpha split with borrowed buffers, the NVMe
+tier, gradient reduce-scatter across ranks. Global-norm clipping cannot be combined with
+stepping during backward (the norm is known only after the last unit) and is not offered here.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+from torch import Tensor
+
+from .memory import RotateContainer, allocate_memory_chunks
+from .optimizer import FlexTrainOptimizer
+from .param_group import StepContextContainer
+
+
+class FlexTrainOptsCoordinator:
+
+    def __init__(self):
+        self._initialized = False
+
+    @property
+    def is_initialized(self) -> bool:
+        return self._initialized
+
+    def _is_invalid_unit(self, unit_index: int) -> bool:
+        return unit_index < 0 or unit_index >= self._num_units
+
+    def _is_invalid_micro_batch(self, micro_batch_index: int) -> bool:
+        return micro_batch_index < 0 or micro_batch_index >= self._micro_batch_per_rank
+
+    def _is_invalid_task(self, unit_index: int, micro_batch_index: int) -> bool:
+        return self._is_invalid_unit(unit_index) or self._is_invalid_micro_batch(micro_batch_index)
+
+    # ------------------------------------------------------------------------------------------
+    def initialize(
+        self,
+        optimizer: FlexTrainOptimizer,
+        unit_half_parameters: Sequence[Tensor],
+        micro_batch_per_rank: int,
+        *,
+        gradacc_dtype: Optional[torch.dtype] = None,
+        offload: bool = True,
+    ) -> None:
+        """
+        Args:
+            optimizer: supplies ``cpu_optimizer`` (the step engine) and ``unit_group_segments``
+                (which parameter group owns which element range of each unit).
+            unit_half_parameters: one flat GPU tensor per unit holding the unit's low-precision
+                parameters, all of the same (padded) length. The update writes new values here.
+            micro_batch_per_rank: number of equal shares a unit's step is cut into; the unit
+                length must be divisible by it.
+            gradacc_dtype: dtype of the gradient buffers (default: the parameters' dtype).
+            offload: master state in pinned host memory (streamed) or resident in HBM.
+        """
+        units = list(unit_half_parameters)
+        assert units and all(t.is_cuda and t.dim() == 1 and t.is_contiguous() for t in units)
+        self._optimizer = optimizer
+        self._num_units = len(units)
+        self._unit_numel = units[0].numel()
+        assert all(t.numel() == self._unit_numel for t in units)
+        assert self._unit_numel % micro_batch_per_rank == 0
+        self._micro_batch_per_rank = micro_batch_per_rank
+        self._unit_half_parameters = units
+        self._offload = bool(offload)
+        device = units[0].device
+        device_dtype = units[0].dtype
+        master_dtype = torch.float32
+        self._emit_half = device_dtype != master_dtype
+        if not self._emit_half:
+            raise NotImplementedError("units must hold fp16 or bf16 parameters; the fp32 master copy is kept beside them")
+        gradacc_dtype = gradacc_dtype or device_dtype
+
+        # Two gradient buffers trade places every unit: [0] receives the unit in backward,
+        # [1] holds the finished gradients of the unit being stepped.
+        self._gpu_bwd_grad_buffers = RotateContainer(tuple(
+            allocate_memory_chunks(self._unit_numel, 2, gradacc_dtype, device)))
+
+        # [master | exp_avg | exp_avg_sq] per unit.
+        per_element = 1 + optimizer.optimizer_state_per_element
+        state_device = torch.device("cpu") if self._offload else device
+        self._unit_opts = allocate_memory_chunks(
+            self._unit_numel, (self._num_units, per_element), master_dtype, state_device)
+
+        # Seed the master copy from the low-precision parameters (exact: widening conversion).
+        for u, half in enumerate(units):
+            self._unit_opts[u][0].copy_(half)
+        if self._offload:
+            torch.cuda.current_stream(device).synchronize()
+
+        # One container per unit: equal shares x parameter groups; every buffer is one piece.
+        n = [self._unit_numel]
+        self._unit_step_ctxts: List[StepContextContainer] = []
+        for u in range(self._num_units):
+            segments = optimizer.unit_group_segments[u]
+            assert segments and segments[-1].end == self._unit_numel, \
+                "unit group segments must cover the padded unit (see FlexTrainOptimizer(aligned_unit_numel=...))"
+            self._unit_step_ctxts.append(StepContextContainer(micro_batch_per_rank, segments, n, n, n))
+        self._initialized = True
+
+    # ---- buffers -------------------------------------------------------------------------------
+    @property
+    def _gpu_bwd_receive_grads(self) -> Tensor:
+        return self._gpu_bwd_grad_buffers[0]
+
+    @property
+    def _gpu_bwd_step_grads(self) -> Tensor:
+        return self._gpu_bwd_grad_buffers[1]
+
+    def unit_master_parameter(self, unit_index: int) -> Tensor:
+        return self._unit_opts[unit_index][0]
+
+    def unit_optimizer_states(self, unit_index: int) -> List[Tensor]:
+        return list(self._unit_opts[unit_index][1:])
+
+    def _rotate_buffers(self) -> None:
+        self._gpu_bwd_grad_buffers.rotate()
+
+    # ---- steps ---------------------------------------------------------------------------------
+    def _plan_optimizer_steps(self, unit_index: int, execute_now: bool = False) -> None:
+        """Bind the unit's step contexts to its buffers (reference ``:605-682``)."""
+        if self._is_invalid_unit(unit_index):
+            return
+        self._unit_step_ctxts[unit_index].plan(
+            half_parameter=self._unit_half_parameters[unit_index],
+            full_parameter=self._unit_opts[unit_index][0],
+            gradient=self._gpu_bwd_step_grads,
+            optimizer_states=[[s] for s in self._unit_opts[unit_index][1:]],
+        )
+        if execute_now:
+            for mb in range(self._micro_batch_per_rank):
+                self._execute_optimizer_step(unit_index, mb)
+
+    def _execute_optimizer_step(self, unit_index: int, micro_batch_index: int) -> None:
+        """Step one micro-batch's share of a unit (reference ``:684-696``). Returns as soon as the
+        work is enqueued."""
+        if self._is_invalid_task(unit_index, micro_batch_index):
+            return
+        contexts = self._unit_step_ctxts[unit_index][micro_batch_index]
+        if self._offload:
+            self._optimizer.cpu_optimizer.step(contexts, blocking=False, guard_stream=False)
+        else:
+            self._optimizer.cpu_optimizer.step(contexts)
+
+    # ---- hooks of the training loop ------------------------------------------------------------
+    def pre_unit_backward(self, unit_index: int) -> Tensor:
+        """Called before the backward pass of ``unit_index`` (units run from last to first).
+        Returns the zeroed buffer the unit's gradients must be accumulated into."""
+        self._rotate_buffers()
+        if self._offload:
+            # The buffer that now receives gradients fed the step of unit_index + 2; its kernels
+            # must have read it before backward overwrites it. A wait on the device, not the host.
+            self._optimizer.cpu_optimizer.stream_wait()
+        self._plan_optimizer_steps(unit_index + 1)
+        receive = self._gpu_bwd_receive_grads
+        receive.zero_()
+        return receive
+
+    def post_micro_batch_backward(self, unit_index: int, micro_batch_index: int) -> None:
+        """Called after each micro-batch's backward of ``unit_index``: steps the same share of the
+        unit that finished before it."""
+        self._execute_optimizer_step(unit_index + 1, micro_batch_index)
+
+    def clear_backward_pipeline(self) -> None:
+        """After the first unit's backward: step it, then wait for everything in flight."""
+        self._rotate_buffers()
+        self._plan_optimizer_steps(0, execute_now=True)
+        self.synchronize()
+
+    def synchronize(self) -> None:
+        if self._offload:
+            self._optimizer.cpu_optimizer.stream_wait()
+            self._optimizer.cpu_optimizer.synchronize()
+        else:
+            torch.cuda.current_stream().synchronize()
+
+
+_OPTS_COORDINATOR = FlexTrainOptsCoordinator()
+
+
+def get_opts_coordinator() -> FlexTrainOptsCoordinator:
+    """Process-wide coordinator (reference ``:891-901``)."""
+    return _OPTS_COORDINATOR

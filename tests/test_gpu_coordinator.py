@@ -1,0 +1,78 @@
+"""GPU test of the per-unit optimizer pipeline: the schedule of the reference's optimizer
+coordinator (step unit u+1 share by share while unit u runs backward) must leave every unit with
+exactly the AdamW result of its accumulated gradient, for resident and offloaded master state."""
+import numpy as np
+import pytest
+import torch
+
+from _util import CODE, HALF_ULP, MASTER_ULP, half_bits, max_ulp, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+class _Unit:
+    def __init__(self, paras):
+        self.paras = paras
+
+
+@pytest.mark.parametrize("offload", [True, False])
+def test_backward_pipeline_matches_oracle(cuda, oracle, offload):
+    from flextrain_amd import FlexTrainAdam
+    from flextrain_amd.coordinator import FlexTrainOptsCoordinator
+    torch.manual_seed(0)
+    num_units, micro_batches, unit_numel = 4, 4, 1 << 20
+    real = unit_numel - 4097  # the tail of each unit is alignment padding
+    # each unit: a weight (decay) and a bias (no decay); the boundary falls inside a share
+    w_numel, b_numel = real - 5000, 5000
+    flat = [torch.zeros(unit_numel, dtype=torch.bfloat16, device=cuda) for _ in range(num_units)]
+    weights, biases = [], []
+    for u in range(num_units):
+        flat[u][:real] = (torch.randn(real, device=cuda) * 0.02).to(torch.bfloat16)
+        weights.append(torch.nn.Parameter(flat[u][:w_numel]))
+        biases.append(torch.nn.Parameter(flat[u][w_numel:real]))
+    decay = {"params": weights, "weight_decay": 0.1}
+    plain = {"params": biases, "weight_decay": 0.0, "lr": 3e-4}
+    opt = FlexTrainAdam([decay, plain], lr=1e-4,
+                        unit_parameter_map={u: _Unit([weights[u], biases[u]]) for u in range(num_units)},
+                        aligned_unit_numel=unit_numel, offload=offload)
+    assert opt.non_layerwise_numel == 0
+    assert [(s.start, s.end) for s in opt.unit_group_segments[0]] == [(0, w_numel), (w_numel, unit_numel)]
+    coord = FlexTrainOptsCoordinator()
+    coord.initialize(opt, flat, micro_batches, offload=offload)
+    assert coord.unit_master_parameter(0).is_pinned() == offload
+
+    # oracle state, seeded the same way
+    state = [(to_np(flat[u].float()).copy(), np.zeros(unit_numel, np.float32), np.zeros(unit_numel, np.float32))
+             for u in range(num_units)]
+    gen = torch.Generator(device=cuda).manual_seed(7)
+    for iteration in (1, 2):
+        opt.update_states()
+        accumulated = {}
+        for u in reversed(range(num_units)):
+            buf = coord.pre_unit_backward(u)
+            for mb in range(micro_batches):
+                g = (torch.randn(unit_numel, device=cuda, generator=gen) * 1e-3).to(torch.bfloat16)
+                g[real:] = 0  # padding never receives gradient
+                buf += g
+                coord.post_micro_batch_backward(u, mb)
+            accumulated[u] = buf.clone()
+        coord.clear_backward_pipeline()
+        for u in range(num_units):
+            pn, mn, vn = state[u]
+            gn = to_np(accumulated[u])
+            hn = np.zeros(unit_numel, np.uint16)
+            for lo, hi, group in ((0, w_numel, decay), (w_numel, unit_numel, plain)):
+                hs = np.zeros(hi - lo, np.uint16)
+                ps, ms, vs = pn[lo:hi].copy(), mn[lo:hi].copy(), vn[lo:hi].copy()
+                oracle.adam_step(ps, np.ascontiguousarray(gn[lo:hi]), ms, vs, step=iteration, lr=group.get("lr", 1e-4),
+                                 weight_decay=group["weight_decay"], g_dtype=CODE[torch.bfloat16], half_out=hs,
+                                 half_dtype=CODE[torch.bfloat16])
+                pn[lo:hi], mn[lo:hi], vn[lo:hi], hn[lo:hi] = ps, ms, vs, hs
+            m, v = coord.unit_optimizer_states(u)
+            worst = dict(p=max_ulp(to_np(coord.unit_master_parameter(u)), pn), m=max_ulp(to_np(m), mn),
+                         v=max_ulp(to_np(v), vn), h=max_ulp(half_bits(flat[u]), hn, bf16=True))
+            print(f"[coordinator offload={offload} it={iteration} unit={u}] worst ULP distance: {worst}", flush=True)
+            assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst["h"] <= HALF_ULP
+    assert decay["step"] == 2 and plain["step"] == 2
+    # the module's parameters are views of the flat unit buffers: they saw the update
+    assert weights[0].data_ptr() == flat[0].data_ptr()
