@@ -207,12 +207,99 @@ def bench_offload(args, torch, dev) -> int:
     return 0 if ok else 3
 
 
+def bench_pipeline(args, torch, dev) -> int:
+    """The per-unit schedule of the optimizer coordinator on Llama-7B layers: while unit u is in
+    backward (here: its synthetic bf16 gradient is copied into the receive buffer, one share per
+    micro-batch), unit u+1 is stepped share by share with its fp32 state streamed from pinned host
+    memory. One step = one pass over all units. No model runs; what is timed is the optimizer side."""
+    import ctypes
+    import gc
+
+    from flextrain_amd import FlexTrainAdam, _C
+    from flextrain_amd.coordinator import FlexTrainOptsCoordinator
+
+    class Unit:
+        def __init__(self, paras):
+            self.paras = paras
+
+    lib = _C.lib()
+    n, mb = N_7B_LAYER, args.micro_batches
+    units = min(args.layers, 24)  # 24 layers = 58 GB of pinned state, inside what the box pins
+    coord = None
+    while coord is None:
+        flat = [(torch.randn(n, device=dev) * 0.02).to(torch.bfloat16) for _ in range(units)]
+        params = [torch.nn.Parameter(f) for f in flat]
+        opt = FlexTrainAdam([{"params": params}], unit_parameter_map={u: Unit([params[u]]) for u in range(units)},
+                            aligned_unit_numel=n, offload=True, **{k: HP[k] for k in ("lr", "betas", "eps", "weight_decay")})
+        opt.cpu_optimizer._offload_chunk = args.chunk_elems
+        opt.cpu_optimizer._offload_slots = args.slots
+        try:
+            coord = FlexTrainOptsCoordinator()
+            coord.initialize(opt, flat, mb, offload=True)
+        except _C.FtError:
+            coord = None
+            del opt, flat, params
+            gc.collect()
+            units -= 2
+            if units < 2:
+                print("cannot pin two layers of optimizer state", file=sys.stderr)
+                return 1
+    grads = (torch.randn(n, device=dev) * 1e-3).to(torch.bfloat16)
+    share = n // mb
+    link = {}
+    out = ctypes.c_double()
+    for name, direction in (("h2d", 0), ("d2h", 1), ("both", 2)):
+        _C.check("ft_link_bandwidth", lib.ft_link_bandwidth(1 << 30, 10, direction, ctypes.byref(out)))
+        link[name] = out.value
+
+    def iteration():
+        opt.update_states()
+        for u in reversed(range(units)):
+            buf = coord.pre_unit_backward(u)
+            for k in range(mb):
+                buf[k * share:(k + 1) * share].copy_(grads[k * share:(k + 1) * share])
+                coord.post_micro_batch_backward(u, k)
+        coord.clear_backward_pipeline()
+
+    for _ in range(args.warmup):
+        iteration()
+    walls = []
+    for _ in range(args.steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        iteration()
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+    sec = sum(walls) / len(walls)
+    total = units * n
+    one_way = total * 12 / sec / 1e9
+    print(json.dumps({
+        "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
+        "value": total / sec, "unit": "elements/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"pipeline: coordinator schedule over {units} Llama-7B layers, {mb} shares per unit, "
+                               "fp32 state in pinned host DRAM, bf16 grads and parameters on GPU",
+                   "elements": total, "units": units, "micro_batches": mb, "chunk_elems": args.chunk_elems,
+                   "slots": args.slots},
+        "link": {"measured_h2d_gbps": link["h2d"], "measured_d2h_gbps": link["d2h"],
+                 "measured_bidirectional_gbps": link["both"], "achieved_each_way_gbps": one_way,
+                 "achieved_total_gbps": 2 * one_way, "frac_of_unidirectional": one_way / min(link["h2d"], link["d2h"]),
+                 "frac_of_bidirectional": 2 * one_way / link["both"]},
+        "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_vec_kernel per share",
+                     "achieved": 2 * one_way, "peak": link["both"], "unit": "GB/s", "frac": 2 * one_way / link["both"],
+                     "traffic": None},
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline"])
+    ap.add_argument("--micro-batches", type=int, default=4, help="pipeline: shares per unit")
     ap.add_argument("--chunk-elems", type=int, default=64 * 1024 * 1024, help="cfg5: elements per streamed chunk")
     ap.add_argument("--slots", type=int, default=3, help="cfg5: device buffer sets of the pipeline")
     ap.add_argument("--layers", type=int, default=32, help="cfg5: decoder layers (32 = the full 7B optimizer)")
@@ -238,6 +325,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if args.workload == "cfg5":
         return bench_offload(args, torch, dev)
+    if args.workload == "pipeline":
+        return bench_pipeline(args, torch, dev)
     eng = FlexTrainCPUAdam(**HP)
 
     if args.workload == "cfg2":

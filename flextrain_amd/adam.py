@@ -62,6 +62,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
         *args,
         offload_chunk_elems: int = DEFAULT_OFFLOAD_CHUNK,
         offload_slots: int = DEFAULT_OFFLOAD_SLOTS,
+        offload_mode: int = 0,
         should_log: bool = False,
         **kwargs,
     ):
@@ -78,6 +79,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
         self._lib = _C.lib()  # raises if the native library is missing: there is no fallback
         self._offload_chunk = int(offload_chunk_elems)
         self._offload_slots = int(offload_slots)
+        self._offload_mode = int(offload_mode)  # FT_OFFLOAD_* of include/ft_adam.h; 0 = automatic
         self._engine: Optional[ctypes.c_void_p] = None
         _C.check("ft_adam_create", self._lib.ft_adam_create(
             self.opt_id, lr, betas[0], betas[1], eps, weight_decay, int(bool(adamw_mode)), int(bool(should_log))))
@@ -106,6 +108,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             handle = ctypes.c_void_p()
             _C.check("ft_offload_create", self._lib.ft_offload_create(
                 self._offload_chunk, self._offload_slots, ctypes.byref(handle)))
+            _C.check("ft_offload_set_mode", self._lib.ft_offload_set_mode(handle, self._offload_mode))
             self._engine = handle
         return self._engine
 

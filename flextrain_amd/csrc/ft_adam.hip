@@ -156,9 +156,13 @@ ftk::AdamConsts make_consts(uint64_t step, float lr, float beta1, float beta2, f
 
 namespace {
 
+struct OutPtrs {
+    float *p, *m, *v;
+};
+
 template <int GT, int HT>
 int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, float* v, void* h, size_t n,
-                 const ft_step_control_t* ctl, hipStream_t stream)
+                 const ft_step_control_t* ctl, hipStream_t stream, OutPtrs out)
 {
     constexpr size_t gsz = (GT == FT_F32) ? 4 : 2;
     const char* gb = reinterpret_cast<const char*>(g);
@@ -172,7 +176,8 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
     size_t head = ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4;
     if (head > n) head = n;
     const bool vec_ok = aligned(mb + head * 4, 16) && aligned(vb + head * 4, 16) &&
-                        aligned(gb + head * gsz, gsz * 4) && (h == nullptr || aligned(hb + head * 2, 8));
+                        aligned(gb + head * gsz, gsz * 4) && (h == nullptr || aligned(hb + head * 2, 8)) &&
+                        aligned(out.p + head, 16) && aligned(out.m + head, 16) && aligned(out.v + head, 16);
     const size_t nvec = vec_ok ? (n - head) / 4 : 0;
     const size_t body = nvec * 4;
 
@@ -183,6 +188,9 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.g = gb + off * gsz;
         a.m = m + off;
         a.v = v + off;
+        a.p_out = out.p + off;
+        a.m_out = out.m + off;
+        a.v_out = out.v + off;
         a.h = h ? hb + off * 2 : nullptr;
         a.ctl = ctl;
         a.n = cnt;
@@ -204,6 +212,9 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.g = gb + head * gsz;
         a.m = m + head;
         a.v = v + head;
+        a.p_out = out.p + head;
+        a.m_out = out.m + head;
+        a.v_out = out.v + head;
         a.h = h ? hb + head * 2 : nullptr;
         a.ctl = ctl;
         a.n = nvec;
@@ -224,17 +235,18 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
 
 template <int GT>
 int launch_g(const ftk::AdamConsts& c, float* p, const void* g, float* m, float* v, void* h, int half_dtype,
-             size_t n, const ft_step_control_t* ctl, hipStream_t stream)
+             size_t n, const ft_step_control_t* ctl, hipStream_t stream, OutPtrs out)
 {
-    if (h == nullptr) return launch_typed<GT, -1>(c, p, g, m, v, nullptr, n, ctl, stream);
-    if (half_dtype == FT_F16) return launch_typed<GT, FT_F16>(c, p, g, m, v, h, n, ctl, stream);
-    return launch_typed<GT, FT_BF16>(c, p, g, m, v, h, n, ctl, stream);
+    if (h == nullptr) return launch_typed<GT, -1>(c, p, g, m, v, nullptr, n, ctl, stream, out);
+    if (half_dtype == FT_F16) return launch_typed<GT, FT_F16>(c, p, g, m, v, h, n, ctl, stream, out);
+    return launch_typed<GT, FT_BF16>(c, p, g, m, v, h, n, ctl, stream, out);
 }
 
 }  // namespace
 
 int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, float* m, float* v,
-                void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream)
+                void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream,
+                float* p_out, float* m_out, float* v_out)
 {
     if (n == 0) return FT_OK;
     if (!p || !g || !m || !v) return fail(FT_EINVAL, "params, grads, exp_avg and exp_avg_sq must not be NULL");
@@ -245,10 +257,13 @@ int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, 
         (half_out && !aligned(half_out, 2)))
         return fail(FT_EALIGN, "a pointer is not aligned to its element size");
     if (ctl && !aligned(ctl, 16)) return fail(FT_EALIGN, "ft_step_control_t must be 16-byte aligned");
+    const OutPtrs out{p_out ? p_out : p, m_out ? m_out : m, v_out ? v_out : v};
+    if (!aligned(out.p, 4) || !aligned(out.m, 4) || !aligned(out.v, 4))
+        return fail(FT_EALIGN, "an output pointer is not aligned to its element size");
     switch (g_dtype) {
-        case FT_F32: return launch_g<FT_F32>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream);
-        case FT_F16: return launch_g<FT_F16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream);
-        default: return launch_g<FT_BF16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream);
+        case FT_F32: return launch_g<FT_F32>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out);
+        case FT_F16: return launch_g<FT_F16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out);
+        default: return launch_g<FT_BF16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out);
     }
 }
 

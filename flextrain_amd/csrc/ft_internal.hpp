@@ -35,8 +35,10 @@ ftk::AdamConsts make_consts(uint64_t step, float lr, float beta1, float beta2, f
                             bool bias_correction, bool adamw_mode, float grad_mult);
 
 // Validates and launches the update over n elements on `stream` (device of the current context).
+// p_out/m_out/v_out: where the new values are written; nullptr = in place.
 int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, float* m, float* v,
-                void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream);
+                void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream,
+                float* p_out = nullptr, float* m_out = nullptr, float* v_out = nullptr);
 
 int cu_count();  // compute units of the current device (cached)
 

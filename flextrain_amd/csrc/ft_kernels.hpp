@@ -152,9 +152,14 @@ __global__ __launch_bounds__(BLOCK) void adam_vec_kernel(AdamArgs a)
     const uint64_t nvec = a.n;
     constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
-    f32x4* __restrict__ P = reinterpret_cast<f32x4*>(a.p);
-    f32x4* __restrict__ M = reinterpret_cast<f32x4*>(a.m);
-    f32x4* __restrict__ V = reinterpret_cast<f32x4*>(a.v);
+    // Inputs and outputs are the same arrays for an in-place update; the offloaded step may point
+    // the outputs elsewhere (staging buffer -> host memory, or the reverse), hence no __restrict__.
+    const f32x4* P = reinterpret_cast<const f32x4*>(a.p);
+    const f32x4* M = reinterpret_cast<const f32x4*>(a.m);
+    const f32x4* V = reinterpret_cast<const f32x4*>(a.v);
+    f32x4* PO = reinterpret_cast<f32x4*>(a.p_out);
+    f32x4* MO = reinterpret_cast<f32x4*>(a.m_out);
+    f32x4* VO = reinterpret_cast<f32x4*>(a.v_out);
 
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         const uint64_t base = tile * kTile + threadIdx.x;
@@ -175,9 +180,9 @@ __global__ __launch_bounds__(BLOCK) void adam_vec_kernel(AdamArgs a)
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
                 const uint64_t i = base + (uint64_t)u * BLOCK;
-                st<NT_ST>(P + i, p[u]);
-                st<NT_ST>(M + i, m[u]);
-                st<NT_ST>(V + i, v[u]);
+                st<NT_ST>(PO + i, p[u]);
+                st<NT_ST>(MO + i, m[u]);
+                st<NT_ST>(VO + i, v[u]);
                 store_h4<HT, NT_ST>(a.h, i, p[u]);
             }
         } else {  // last, partial tile
@@ -187,9 +192,9 @@ __global__ __launch_bounds__(BLOCK) void adam_vec_kernel(AdamArgs a)
                 f32x4 gg = load_g4<GT, false>(a.g, i);
                 f32x4 pp = P[i], mm = M[i], vv = V[i];
                 adam_unit(pp, gg, mm, vv, c);
-                P[i] = pp;
-                M[i] = mm;
-                V[i] = vv;
+                PO[i] = pp;
+                MO[i] = mm;
+                VO[i] = vv;
                 store_h4<HT, false>(a.h, i, pp);
             }
         }
@@ -215,9 +220,9 @@ __global__ __launch_bounds__(256) void adam_scalar_kernel(AdamArgs a)
             g = half_to_float<GT>(reinterpret_cast<const uint16_t*>(a.g)[i]);
         float p = a.p[i], m = a.m[i], v = a.v[i];
         adam_element(p, g, m, v, c);
-        a.p[i] = p;
-        a.m[i] = m;
-        a.v[i] = v;
+        a.p_out[i] = p;
+        a.m_out[i] = m;
+        a.v_out[i] = v;
         if constexpr (HT == FT_F16 || HT == FT_BF16)
             reinterpret_cast<uint16_t*>(a.h)[i] = (uint16_t)(pack2<HT>(p, 0.0f) & 0xffffu);
     }

@@ -23,6 +23,7 @@ struct Slot {
     void* g = nullptr;  // staging for host-resident gradients (chunk * 4 bytes), lazily allocated
     void* h = nullptr;  // staging for a host-resident low-precision copy (chunk * 2 bytes), lazy
     hipEvent_t h2d_done = nullptr, k_done = nullptr, d2h_done = nullptr;
+    hipEvent_t free_ev = nullptr;  // whichever of the above marks the slot's last use
     bool used = false;
 };
 
@@ -42,6 +43,12 @@ struct Pending {
 
 constexpr size_t kMaxPending = 8;
 
+// Automatic choice of the transfer mode. Measured on MI355X / PCIe Gen5 x16: SDMA copies through
+// staging slots move 48-49 GB/s each way when every copy is at least ~128 MiB, but a run of many
+// smaller copies ends up with both directions on one SDMA engine and drops to 15 GB/s; the kernel
+// reading and writing pinned host memory itself holds 45 GB/s each way at any size.
+constexpr size_t kStagedMinElems = 32u * 1024u * 1024u;
+
 struct Engine {
     uint32_t magic = 0x46544f45;  // "FTOE"
     int device = 0;
@@ -53,6 +60,8 @@ struct Engine {
     hipEvent_t ev_end = nullptr;    // last D2H of the last step
     hipEvent_t ev_kernels = nullptr;  // last kernel of the last step
     bool stepped = false;
+    size_t cursor = 0;  // chunks enqueued so far; slots are taken round-robin across steps
+    int mode = FT_OFFLOAD_AUTO;
     std::deque<Pending> recent;        // steps whose write-back may still be in flight, oldest first
     std::vector<hipEvent_t> free_events;
 };
@@ -207,13 +216,6 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
 
     const size_t gsz = g_dtype == FT_F32 ? 4 : 2;
     const size_t chunk = e->chunk;
-    if (g_on_host || (half_out && half_on_host)) {
-        for (Slot& s : e->slots) {
-            if (g_on_host && !s.g) FT_HIP(hipMalloc(&s.g, chunk * 4));
-            if (half_out && half_on_host && !s.h) FT_HIP(hipMalloc(&s.h, chunk * 2));
-        }
-    }
-
     const ftk::AdamConsts c =
         fth::make_consts(step, lr, beta1, beta2, eps, weight_decay, bias_correction != 0, o.adamw_mode, grad_mult);
     hipStream_t user = static_cast<hipStream_t>(stream);
@@ -241,6 +243,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     for (auto it = e->recent.rbegin(); it != e->recent.rend(); ++it) {
         if (it->overlaps(mine)) {
             FT_HIP(hipStreamWaitEvent(e->s_h2d, it->done, 0));
+            FT_HIP(hipStreamWaitEvent(e->s_k, it->done, 0));
             break;
         }
     }
@@ -252,37 +255,73 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     const char* gb = static_cast<const char*>(g);
     char* hb = static_cast<char*>(half_out);
 
-    size_t ci = 0;
-    for (size_t off = 0; off < n; off += chunk, ++ci) {
+    // How the state crosses the link (see ft_offload_set_mode). Staged = SDMA copy through a device
+    // buffer slot; direct = the update kernel itself reads or writes the pinned host arrays.
+    int mode = e->mode;
+    if (mode == FT_OFFLOAD_AUTO) mode = (n >= kStagedMinElems) ? FT_OFFLOAD_STAGED : FT_OFFLOAD_DIRECT;
+    const bool in_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_IN;
+    const bool out_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_OUT;
+    const bool stage_g = g_on_host && in_staged;
+    const bool stage_h = half_out && half_on_host && out_staged;
+    for (Slot& s : e->slots) {
+        if (stage_g && !s.g) FT_HIP(hipMalloc(&s.g, chunk * 4));
+        if (stage_h && !s.h) FT_HIP(hipMalloc(&s.h, chunk * 2));
+    }
+
+    for (size_t off = 0; off < n; off += chunk) {
         const size_t cnt = (n - off < chunk) ? (n - off) : chunk;
-        Slot& s = e->slots[ci % e->slots.size()];
-
-        if (s.used) FT_HIP(hipStreamWaitEvent(e->s_h2d, s.d2h_done, 0));
-        FT_HIP(hipMemcpyAsync(s.p, hp + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
-        FT_HIP(hipMemcpyAsync(s.m, hm + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
-        FT_HIP(hipMemcpyAsync(s.v, hv + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
-        if (g_on_host) FT_HIP(hipMemcpyAsync(s.g, gb + off * gsz, cnt * gsz, hipMemcpyHostToDevice, e->s_h2d));
-        FT_HIP(hipEventRecord(s.h2d_done, e->s_h2d));
-
-        FT_HIP(hipStreamWaitEvent(e->s_k, s.h2d_done, 0));
-        const void* kg = g_on_host ? s.g : static_cast<const void*>(gb + off * gsz);
-        void* kh = nullptr;
-        if (half_out) kh = half_on_host ? s.h : static_cast<void*>(hb + off * 2);
-        rc = fth::launch_adam(c, s.p, kg, g_dtype, s.m, s.v, kh, half_dtype, cnt,
-                              static_cast<const ft_step_control_t*>(ctl), e->s_k);
+        float *kp = hp + off, *km = hm + off, *kv = hv + off;          // kernel inputs
+        float *op = hp + off, *om = hm + off, *ov = hv + off;          // kernel outputs
+        const void* kg = gb + off * gsz;
+        void* kh = half_out ? static_cast<void*>(hb + off * 2) : nullptr;
+        Slot* slot = nullptr;
+        if (in_staged || out_staged) {
+            // Round-robin over all steps, not per step: a step that is a single chunk (one share
+            // of a unit) must not queue behind the previous step's last use of the same slot.
+            slot = &e->slots[e->cursor++ % e->slots.size()];
+            if (slot->used) FT_HIP(hipStreamWaitEvent(in_staged ? e->s_h2d : e->s_k, slot->free_ev, 0));
+        }
+        if (in_staged) {
+            FT_HIP(hipMemcpyAsync(slot->p, hp + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
+            FT_HIP(hipMemcpyAsync(slot->m, hm + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
+            FT_HIP(hipMemcpyAsync(slot->v, hv + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
+            if (stage_g) {
+                FT_HIP(hipMemcpyAsync(slot->g, gb + off * gsz, cnt * gsz, hipMemcpyHostToDevice, e->s_h2d));
+                kg = slot->g;
+            }
+            FT_HIP(hipEventRecord(slot->h2d_done, e->s_h2d));
+            FT_HIP(hipStreamWaitEvent(e->s_k, slot->h2d_done, 0));
+            kp = slot->p;
+            km = slot->m;
+            kv = slot->v;
+        }
+        if (out_staged) {
+            op = slot->p;
+            om = slot->m;
+            ov = slot->v;
+            if (stage_h) kh = slot->h;
+        }
+        rc = fth::launch_adam(c, kp, kg, g_dtype, km, kv, kh, half_dtype, cnt,
+                              static_cast<const ft_step_control_t*>(ctl), e->s_k, op, om, ov);
         if (rc != FT_OK) return rc;
-        FT_HIP(hipEventRecord(s.k_done, e->s_k));
-
-        FT_HIP(hipStreamWaitEvent(e->s_d2h, s.k_done, 0));
-        FT_HIP(hipMemcpyAsync(hp + off, s.p, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
-        FT_HIP(hipMemcpyAsync(hm + off, s.m, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
-        FT_HIP(hipMemcpyAsync(hv + off, s.v, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
-        if (half_out && half_on_host)
-            FT_HIP(hipMemcpyAsync(hb + off * 2, s.h, cnt * 2, hipMemcpyDeviceToHost, e->s_d2h));
-        FT_HIP(hipEventRecord(s.d2h_done, e->s_d2h));
-        s.used = true;
+        if (slot) {
+            FT_HIP(hipEventRecord(slot->k_done, e->s_k));
+            slot->free_ev = slot->k_done;
+            slot->used = true;
+        }
+        if (out_staged) {
+            FT_HIP(hipStreamWaitEvent(e->s_d2h, slot->k_done, 0));
+            FT_HIP(hipMemcpyAsync(hp + off, slot->p, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
+            FT_HIP(hipMemcpyAsync(hm + off, slot->m, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
+            FT_HIP(hipMemcpyAsync(hv + off, slot->v, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
+            if (stage_h) FT_HIP(hipMemcpyAsync(hb + off * 2, slot->h, cnt * 2, hipMemcpyDeviceToHost, e->s_d2h));
+            FT_HIP(hipEventRecord(slot->d2h_done, e->s_d2h));
+            slot->free_ev = slot->d2h_done;
+        }
     }
     FT_HIP(hipEventRecord(e->ev_kernels, e->s_k));
+    // the write-back is complete when the D2H stream is, and (direct output) when the kernels are
+    FT_HIP(hipStreamWaitEvent(e->s_d2h, e->ev_kernels, 0));
     FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
     e->stepped = true;
 
@@ -291,6 +330,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     if (e->free_events.empty()) {
         Pending& old = e->recent.front();
         FT_HIP(hipStreamWaitEvent(e->s_h2d, old.done, 0));
+        FT_HIP(hipStreamWaitEvent(e->s_k, old.done, 0));
         e->free_events.push_back(old.done);
         e->recent.pop_front();
     }
@@ -298,6 +338,15 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     e->free_events.pop_back();
     FT_HIP(hipEventRecord(mine.done, e->s_d2h));
     e->recent.push_back(mine);
+    return FT_OK;
+}
+
+int ft_offload_set_mode(void* handle, int mode)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    if (mode < FT_OFFLOAD_AUTO || mode > FT_OFFLOAD_STAGED_OUT) return fth::fail(FT_EINVAL, "unknown offload mode %d", mode);
+    e->mode = mode;
     return FT_OK;
 }
 

@@ -17,10 +17,13 @@ struct AdamConsts {
 };
 
 struct AdamArgs {
-    float* p;
+    const float* p;  // inputs ...
     const void* g;
-    float* m;
-    float* v;
+    const float* m;
+    const float* v;
+    float* p_out;    // ... and where the new values go (the same arrays for an in-place update)
+    float* m_out;
+    float* v_out;
     void* h;                       // low-precision copy or nullptr
     const ft_step_control_t* ctl;  // device decision or nullptr
     uint64_t n;                    // elements (scalar kernel) or 4-element units (vector kernel)

@@ -140,7 +140,16 @@ int ft_pinned_free(void* ptr);
  * ft_offload_elapsed_ms: device time between the first H2D and the last D2H of the last
  *                    enqueued step (waits for it).
  */
+enum {
+    FT_OFFLOAD_AUTO = 0,       /* staged for steps of at least 32 Mi elements, direct for shorter ones */
+    FT_OFFLOAD_STAGED = 1,     /* SDMA H2D into a slot, kernel in place on the slot, SDMA D2H            */
+    FT_OFFLOAD_DIRECT = 2,     /* no copies: the kernel reads and writes the pinned host arrays itself   */
+    FT_OFFLOAD_STAGED_IN = 3,  /* SDMA H2D into a slot, the kernel writes its results to host memory     */
+    FT_OFFLOAD_STAGED_OUT = 4  /* the kernel reads host memory, results leave through a slot and SDMA D2H */
+};
 int ft_offload_create(size_t chunk_elems, int n_slots, void** out_handle);
+/* How the state crosses the host link; results are identical in every mode. */
+int ft_offload_set_mode(void* handle, int mode);
 int ft_offload_destroy(void* handle);
 int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, float beta2,
                     float eps, float weight_decay, int bias_correction, float grad_mult,

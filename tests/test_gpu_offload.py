@@ -92,11 +92,11 @@ def test_data_stream_orders_copies_behind_their_producer(cuda):
 
 @pytest.mark.parametrize("slots", [2, 3])
 @pytest.mark.parametrize("n,chunk", [(1_000_003, 1 << 16), (300_000, 1 << 20), (4 * (1 << 16), 1 << 16)])
-def test_streamed_step_device_grads(cuda, oracle, n, chunk, slots):
+def test_streamed_step_device_grads(cuda, oracle, n, chunk, slots, mode=1):
     """Master state in pinned host memory, bf16 grads and bf16 copy on the GPU (the offloaded
     configuration), several chunks, ragged last chunk, two steps in a row."""
     from flextrain_amd import FlexTrainCPUAdam
-    eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=slots, **HP)
+    eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=slots, offload_mode=mode, **HP)
     p, m, v = _host_state(n, seed=n)
     h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
     gen = torch.Generator(device=cuda).manual_seed(1)
@@ -107,13 +107,14 @@ def test_streamed_step_device_grads(cuda, oracle, n, chunk, slots):
         _assert_equal_bits(f"offload n={n} chunk={chunk} slots={slots} t={t}", p, m, v, h, want, torch.bfloat16)
 
 
-def test_streamed_step_reference_layout(cuda, oracle):
+@pytest.mark.parametrize("mode", [1, 2, 3, 4])
+def test_streamed_step_reference_layout(cuda, oracle, mode):
     """Everything in pinned host memory with fp32 gradients and an fp16 copy: the layout the
     reference's coordinator hands to the step."""
     from flextrain_amd import FlexTrainCPUAdam
     from flextrain_amd.memory import pinned_empty
     n = 700_001
-    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 17, offload_slots=2, **HP)
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 17, offload_slots=2, offload_mode=mode, **HP)
     p, m, v = _host_state(n, seed=3)
     g = pinned_empty(n, torch.float32)
     g.copy_(torch.randn(n) * 1e-3)
@@ -125,10 +126,13 @@ def test_streamed_step_reference_layout(cuda, oracle):
     assert eng.last_offload_ms() > 0
 
 
-def test_streamed_equals_resident_bit_for_bit(cuda):
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+def test_streamed_equals_resident_bit_for_bit(cuda, mode):
+    """Every transfer mode (automatic, staged, direct, staged-in, staged-out) gives the resident
+    kernel's bits."""
     from flextrain_amd import FlexTrainCPUAdam
     n = 3_000_017
-    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 18, offload_slots=3, **HP)
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 18, offload_slots=3, offload_mode=mode, **HP)
     p, m, v = _host_state(n, seed=8)
     g = (torch.randn(n, device=cuda) * 1e-3 * 512).to(torch.float16)
     dp, dm, dv = p.to(cuda), m.to(cuda), v.to(cuda)
@@ -174,13 +178,14 @@ def test_link_probe_reports_sane_numbers(cuda):
         assert 1.0 < out.value < 1000.0
 
 
-def test_steps_on_disjoint_memory_overlap_and_same_memory_stay_ordered(cuda, oracle):
+@pytest.mark.parametrize("mode", [1, 2, 3, 4])
+def test_steps_on_disjoint_memory_overlap_and_same_memory_stay_ordered(cuda, oracle, mode):
     """Per-unit use: many non-blocking steps in a row, each on its own host arrays, then two on the
     same arrays; every result must equal the oracle's, and more steps than the engine tracks
     individually (8) must still be ordered correctly."""
     from flextrain_amd import FlexTrainCPUAdam
     n, units = 400_000, 12
-    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 17, offload_slots=2, **HP)
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 17, offload_slots=2, offload_mode=mode, **HP)
     state = [_host_state(n, seed=50 + u) for u in range(units)]
     grads = [(torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16) for _ in range(units)]
     halves = [torch.zeros(n, dtype=torch.bfloat16, device=cuda) for _ in range(units)]
