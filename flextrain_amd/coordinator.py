@@ -93,11 +93,21 @@ class FlexTrainOptsCoordinator:
         if not self._emit_half:
             raise NotImplementedError("units must hold fp16 or bf16 parameters; the fp32 master copy is kept beside them")
         gradacc_dtype = gradacc_dtype or device_dtype
+        self._gradacc_dtype_incompatible = gradacc_dtype != device_dtype
 
         # Two gradient buffers trade places every unit: [0] receives the unit in backward,
         # [1] holds the finished gradients of the unit being stepped.
         self._gpu_bwd_grad_buffers = RotateContainer(tuple(
             allocate_memory_chunks(self._unit_numel, 2, gradacc_dtype, device)))
+        # When gradients are accumulated in a wider type than backward produces them in, backward
+        # writes each micro-batch into this extra buffer and one fused pass per micro-batch adds it
+        # to the receive buffer and clears it (reference ``:187-190,743,775-777``: a zero_ before
+        # and a += after every micro-batch).
+        self._gpu_bwd_extra_grads = None
+        if self._gradacc_dtype_incompatible:
+            from .loss_scaler import GradientGuard
+            self._gpu_bwd_extra_grads = allocate_memory_chunks(self._unit_numel, 1, device_dtype, device)[0]
+            self._guard = GradientGuard(device)
 
         # [master | exp_avg | exp_avg_sq] per unit.
         per_element = 1 + optimizer.optimizer_state_per_element
@@ -168,7 +178,9 @@ class FlexTrainOptsCoordinator:
     # ---- hooks of the training loop ------------------------------------------------------------
     def pre_unit_backward(self, unit_index: int) -> Tensor:
         """Called before the backward pass of ``unit_index`` (units run from last to first).
-        Returns the zeroed buffer the unit's gradients must be accumulated into."""
+        Returns the zeroed buffer backward must write the unit's gradients into: the accumulation
+        buffer itself (backward accumulates over micro-batches), or -- when accumulation happens in
+        a wider type -- the buffer for one micro-batch's gradients."""
         self._rotate_buffers()
         if self._offload:
             # The buffer that now receives gradients fed the step of unit_index + 2; its kernels
@@ -177,11 +189,14 @@ class FlexTrainOptsCoordinator:
         self._plan_optimizer_steps(unit_index + 1)
         receive = self._gpu_bwd_receive_grads
         receive.zero_()
-        return receive
+        return self._gpu_bwd_extra_grads if self._gradacc_dtype_incompatible else receive
 
     def post_micro_batch_backward(self, unit_index: int, micro_batch_index: int) -> None:
-        """Called after each micro-batch's backward of ``unit_index``: steps the same share of the
-        unit that finished before it."""
+        """Called after each micro-batch's backward of ``unit_index``: folds the micro-batch's
+        gradients into the accumulation buffer when the two differ in type, then steps the same
+        share of the unit that finished before it."""
+        if self._gradacc_dtype_incompatible:
+            self._guard.accumulate(self._gpu_bwd_receive_grads, self._gpu_bwd_extra_grads, zero_grads=True)
         self._execute_optimizer_step(unit_index + 1, micro_batch_index)
 
     def clear_backward_pipeline(self) -> None:

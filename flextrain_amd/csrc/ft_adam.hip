@@ -41,6 +41,9 @@
 #ifndef FT_STATS_UNROLL
 #define FT_STATS_UNROLL 4
 #endif
+#ifndef FT_ACCUM_WAVES_PER_CU
+#define FT_ACCUM_WAVES_PER_CU 12
+#endif
 #ifndef FT_STATS_BLOCKS_PER_CU
 #define FT_STATS_BLOCKS_PER_CU 4
 #endif
@@ -56,6 +59,7 @@ std::unordered_map<int, void*> g_stats_ws;    // device -> library-owned statist
 int g_adam_waves_per_cu = FT_ADAM_WAVES_PER_CU;
 std::unordered_map<int, int> g_lds_per_cu;   // device -> bytes of LDS per compute unit
 int g_stats_blocks_per_cu = FT_STATS_BLOCKS_PER_CU;
+int g_accum_waves_per_cu = FT_ACCUM_WAVES_PER_CU;
 
 constexpr int kMaxStatsBlocks = 8192;
 
@@ -100,16 +104,19 @@ int cu_count()
     return n;
 }
 
-// Dynamic LDS requested per workgroup of the update kernel. The kernel never touches it: the
-// allocation only bounds how many workgroups fit on a compute unit at once.
-unsigned adam_throttle_lds_bytes()
+// Dynamic LDS requested per 64-lane workgroup of a streaming kernel. The kernel never touches it:
+// the allocation only bounds how many workgroups fit on a compute unit at once. The tuned figure
+// (g_adam_waves_per_cu) is for the update with 16-bit gradients, whose lanes have 56 bytes of loads
+// in flight each; what has to stay constant is the bytes in flight per compute unit, so a kernel
+// that loads fewer bytes per lane gets proportionally more resident wavefronts.
+unsigned throttle_lds_bytes(unsigned load_bytes_per_lane)
 {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 0;
     std::lock_guard<std::mutex> lk(g_mu);
-    const int waves = g_adam_waves_per_cu;
-    constexpr int kMaxResident = 32 * 64 / FT_ADAM_BLOCK;  // hardware limit: 32 wavefronts per CU
-    if (waves >= kMaxResident) return 0;
+    int waves = (g_adam_waves_per_cu * 56 + static_cast<int>(load_bytes_per_lane) / 2) / static_cast<int>(load_bytes_per_lane);
+    if (waves < 1) waves = 1;
+    if (waves >= 32) return 0;  // hardware limit: 32 wavefronts per CU anyway
     auto it = g_lds_per_cu.find(dev);
     int lds = 0;
     if (it != g_lds_per_cu.end()) {
@@ -225,7 +232,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         if (blocks > cap) blocks = cap;
         hipLaunchKernelGGL(
             (ftk::adam_vec_kernel<GT, HT, FT_ADAM_BLOCK, FT_ADAM_UNROLL, FT_ADAM_NT_LD, FT_ADAM_NT_ST>),
-            dim3(static_cast<unsigned>(blocks)), dim3(FT_ADAM_BLOCK), adam_throttle_lds_bytes(), stream, a);
+            dim3(static_cast<unsigned>(blocks)), dim3(FT_ADAM_BLOCK), throttle_lds_bytes(48 + 4 * static_cast<unsigned>(gsz)), stream, a);
         FT_HIP(hipGetLastError());
     }
     int rc = scalar_part(0, head);
@@ -272,6 +279,91 @@ int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, 
 // ================================================================================================
 // C ABI
 // ================================================================================================
+extern "C" size_t ft_grad_stats_workspace_bytes(void);
+
+namespace {
+
+// The caller's scratch if given (checked), else the per-device buffer the library owns.
+int resolve_stats_workspace(void* workspace, size_t workspace_bytes, ftk::StatsPartial** out)
+{
+    ftk::StatsPartial* parts = static_cast<ftk::StatsPartial*>(workspace);
+    if (parts) {
+        if (workspace_bytes < ft_grad_stats_workspace_bytes())
+            return fth::fail(FT_EINVAL, "workspace of %zu bytes is smaller than ft_grad_stats_workspace_bytes()",
+                             workspace_bytes);
+        if (!aligned(parts, 16)) return fth::fail(FT_EALIGN, "workspace must be 16-byte aligned");
+    } else {
+        int dev = 0;
+        FT_HIP(hipGetDevice(&dev));
+        std::lock_guard<std::mutex> lk(g_mu);
+        auto it = g_stats_ws.find(dev);
+        if (it == g_stats_ws.end()) {
+            void* w = nullptr;
+            FT_HIP(hipMalloc(&w, ft_grad_stats_workspace_bytes()));
+            g_stats_ws[dev] = w;
+            parts = static_cast<ftk::StatsPartial*>(w);
+        } else {
+            parts = static_cast<ftk::StatsPartial*>(it->second);
+        }
+    }
+    *out = parts;
+    return FT_OK;
+}
+
+template <int AT, int GT, bool ZERO, bool STATS>
+int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, float scale, float pre_mult,
+                      ftk::StatsPartial* parts, int blocks, hipStream_t stream)
+{
+    constexpr size_t asz = (AT == FT_F32) ? 4 : 2, gsz = (GT == FT_F32) ? 4 : 2;
+    if (nvec > 0) {
+        // Without statistics there are no per-block partials to bound, so the kernel runs like the
+        // update: one tile per wavefront-sized workgroup, residency throttled through dynamic LDS.
+        unsigned lds = 0;
+        if (!STATS) {
+            size_t b = (nvec + 63) / 64;
+            if (b > 0x7fffffffu) b = 0x7fffffffu;
+            blocks = static_cast<int>(b);
+            lds = fth::throttle_lds_bytes(4 * static_cast<unsigned>(asz + gsz));
+        }
+        hipLaunchKernelGGL((ftk::grad_accumulate_kernel<AT, GT, ZERO, STATS, 64>), dim3(blocks), dim3(64), lds, stream,
+                           static_cast<void*>(static_cast<char*>(acc) + head * asz),
+                           static_cast<void*>(static_cast<char*>(g) + head * gsz), static_cast<uint64_t>(nvec), scale,
+                           pre_mult, parts);
+        FT_HIP(hipGetLastError());
+    }
+    const size_t tail_begin = head + nvec * 4;
+    if (STATS || head > 0 || tail_begin < n) {
+        hipLaunchKernelGGL((ftk::grad_accumulate_edge_kernel<AT, GT, ZERO, STATS>), dim3(1), dim3(64), 0, stream, acc, g,
+                           static_cast<uint64_t>(head), static_cast<uint64_t>(tail_begin), static_cast<uint64_t>(n),
+                           scale, pre_mult, parts + blocks);
+        FT_HIP(hipGetLastError());
+    }
+    return FT_OK;
+}
+
+template <int AT, int GT>
+int launch_accumulate_flags(bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec, float scale,
+                            float pre_mult, ftk::StatsPartial* parts, int blocks, hipStream_t stream)
+{
+    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+}
+
+template <int AT>
+int launch_accumulate_g(int g_dtype, bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec,
+                        float scale, float pre_mult, ftk::StatsPartial* parts, int blocks, hipStream_t stream)
+{
+    switch (g_dtype) {
+        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+    }
+}
+
+}  // namespace
+
 extern "C" {
 
 const char* ft_last_error(void) { return t_last_error.c_str(); }
@@ -339,26 +431,9 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
     if (n > 0 && !g) return fth::fail(FT_EINVAL, "g must not be NULL");
     if (n > 0 && !aligned(g, elem_size(g_dtype))) return fth::fail(FT_EALIGN, "g is not aligned to its element size");
 
-    ftk::StatsPartial* parts = static_cast<ftk::StatsPartial*>(workspace);
-    if (parts) {
-        if (workspace_bytes < ft_grad_stats_workspace_bytes())
-            return fth::fail(FT_EINVAL, "workspace of %zu bytes is smaller than ft_grad_stats_workspace_bytes()",
-                             workspace_bytes);
-        if (!aligned(parts, 16)) return fth::fail(FT_EALIGN, "workspace must be 16-byte aligned");
-    } else {
-        int dev = 0;
-        FT_HIP(hipGetDevice(&dev));
-        std::lock_guard<std::mutex> lk(g_mu);
-        auto it = g_stats_ws.find(dev);
-        if (it == g_stats_ws.end()) {
-            void* w = nullptr;
-            FT_HIP(hipMalloc(&w, ft_grad_stats_workspace_bytes()));
-            g_stats_ws[dev] = w;
-            parts = static_cast<ftk::StatsPartial*>(w);
-        } else {
-            parts = static_cast<ftk::StatsPartial*>(it->second);
-        }
-    }
+    ftk::StatsPartial* parts = nullptr;
+    int wrc = resolve_stats_workspace(workspace, workspace_bytes, &parts);
+    if (wrc != FT_OK) return wrc;
 
     const size_t esz = elem_size(g_dtype);
     const size_t per_unit = 16 / esz;
@@ -413,6 +488,56 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
     return FT_OK;
 }
 
+int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                       float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
+                       size_t workspace_bytes, void* stream_)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (!valid_dtype(acc_dtype) || !valid_dtype(g_dtype))
+        return fth::fail(FT_EINVAL, "unknown dtype code (acc %d, g %d)", acc_dtype, g_dtype);
+    if (stats_out && !aligned(stats_out, 16)) return fth::fail(FT_EALIGN, "ft_grad_stats_t must be 16-byte aligned");
+    const bool stats = stats_out != nullptr;
+    if (n > 0 && (!acc || !g)) return fth::fail(FT_EINVAL, "acc and g must not be NULL");
+    const size_t asz = elem_size(acc_dtype), gsz = elem_size(g_dtype);
+    size_t head = 0, nvec = 0;
+    if (n > 0) {
+        if (!aligned(acc, asz) || !aligned(g, gsz)) return fth::fail(FT_EALIGN, "a pointer is not aligned to its element size");
+        head = ((asz * 4 - (reinterpret_cast<uintptr_t>(acc) & (asz * 4 - 1))) & (asz * 4 - 1)) / asz;
+        if (head > n) head = n;
+        if (!aligned(static_cast<char*>(g) + head * gsz, gsz * 4))
+            return fth::fail(FT_EALIGN, "acc and g must start at the same element offset modulo 4 of their buffers");
+        nvec = (n - head) / 4;
+    }
+    ftk::StatsPartial* parts = nullptr;
+    if (stats) {
+        int wrc = resolve_stats_workspace(workspace, workspace_bytes, &parts);
+        if (wrc != FT_OK) return wrc;
+    }
+    int blocks = 0;
+    if (nvec > 0) {
+        size_t b = (nvec + 63) / 64;  // one wavefront per workgroup, a persistent grid of them
+        size_t cap = static_cast<size_t>(fth::cu_count()) * static_cast<size_t>(g_accum_waves_per_cu);
+        if (cap > static_cast<size_t>(kMaxStatsBlocks - 1)) cap = kMaxStatsBlocks - 1;
+        if (b > cap) b = cap;
+        blocks = static_cast<int>(b);
+    }
+    int rc;
+    switch (acc_dtype) {
+        case FT_F32: rc = launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, blocks, stream); break;
+        case FT_F16: rc = launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, blocks, stream); break;
+        default: rc = launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, blocks, stream); break;
+    }
+    if (rc != FT_OK) return rc;
+    if (stats) {
+        // block partials [0, blocks) plus the edge kernel's one at index `blocks`
+        hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, blocks + 1,
+                           static_cast<const void*>(nullptr), static_cast<uint64_t>(0), static_cast<uint64_t>(0),
+                           static_cast<uint64_t>(0), 1.0f, static_cast<ft_grad_stats_t*>(stats_out), stats_accumulate);
+        FT_HIP(hipGetLastError());
+    }
+    return FT_OK;
+}
+
 int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ctl_out, void* stream)
 {
     if (!stats || !ctl_out) return fth::fail(FT_EINVAL, "stats and ctl_out must not be NULL");
@@ -425,9 +550,10 @@ int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ct
     return FT_OK;
 }
 
-int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu)
+int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu, int accumulate_waves_per_cu)
 {
     std::lock_guard<std::mutex> lk(g_mu);
+    g_accum_waves_per_cu = accumulate_waves_per_cu > 0 ? accumulate_waves_per_cu : FT_ACCUM_WAVES_PER_CU;
     g_adam_waves_per_cu = adam_waves_per_cu > 0 ? adam_waves_per_cu : FT_ADAM_WAVES_PER_CU;
     g_stats_blocks_per_cu = stats_blocks_per_cu > 0 ? stats_blocks_per_cu : FT_STATS_BLOCKS_PER_CU;
     return FT_OK;

@@ -42,4 +42,8 @@ int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, 
 
 int cu_count();  // compute units of the current device (cached)
 
+// Dynamic LDS per 64-lane workgroup that keeps the bytes in flight per CU at the tuned level for a
+// kernel whose lanes each have `load_bytes_per_lane` bytes of loads outstanding.
+unsigned throttle_lds_bytes(unsigned load_bytes_per_lane);
+
 }  // namespace fth

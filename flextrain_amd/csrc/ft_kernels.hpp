@@ -295,6 +295,35 @@ __device__ __forceinline__ void stats_accumulate(u32x4 w, float pre_mult, float 
     }
 }
 
+// Block-level end of a statistics pass: per-lane fp32 sums and counts -> one fp64 partial per block.
+template <int BLOCK>
+__device__ __forceinline__ void block_stats_epilogue(const float (&acc)[4], uint32_t bad, StatsPartial* __restrict__ partials)
+{
+    const float t = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+    const uint32_t tb = wave_sum_u32(bad);
+
+    constexpr int kWaves = BLOCK / kWave;
+    __shared__ float s_sum[kWaves];
+    __shared__ uint32_t s_bad[kWaves];
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        s_sum[wave] = t;
+        s_bad[wave] = tb;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double s = 0.0;
+        uint64_t b = 0;
+#pragma unroll
+        for (int k = 0; k < kWaves; ++k) {
+            s += (double)s_sum[k];
+            b += s_bad[k];
+        }
+        partials[blockIdx.x].sumsq = s;
+        partials[blockIdx.x].nonfinite = b;
+    }
+}
+
 // Stage 1: every block writes one StatsPartial. nvec = number of 16-byte units; the caller
 // handles the elements outside [0, nvec*per_unit) in grad_stats_final_kernel.
 template <int GT, int BLOCK, int UNROLL>
@@ -321,29 +350,7 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
             }
         }
     }
-    const float t = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
-    const uint32_t tb = wave_sum_u32(bad);
-
-    constexpr int kWaves = BLOCK / kWave;
-    __shared__ float s_sum[kWaves];
-    __shared__ uint32_t s_bad[kWaves];
-    const int wave = threadIdx.x / kWave;
-    if ((threadIdx.x & (kWave - 1)) == 0) {
-        s_sum[wave] = t;
-        s_bad[wave] = tb;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        double s = 0.0;
-        uint64_t b = 0;
-#pragma unroll
-        for (int k = 0; k < kWaves; ++k) {
-            s += (double)s_sum[k];
-            b += s_bad[k];
-        }
-        partials[blockIdx.x].sumsq = s;
-        partials[blockIdx.x].nonfinite = b;
-    }
+    block_stats_epilogue<BLOCK>(acc, bad, partials);
 }
 
 // Stage 2 (one block of 256): adds the block partials in a fixed tree order, then the up to
@@ -404,6 +411,141 @@ __global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartia
             out->sumsq = s;
             out->nonfinite = b;
         }
+    }
+}
+
+// ---- gradient accumulation ---------------------------------------------------------------------
+// acc[i] = fma((float)g[i], scale, acc[i]), rounded to acc's type (scale == 1 is a plain add of the
+// widened gradient). Optionally clears g afterwards and gathers the statistics of the new acc
+// (exactly what grad_stats_kernel would report for it), so that the pass over the gradients that
+// accumulation needs anyway also yields the overflow flag and the norm.
+template <int AT>
+__device__ __forceinline__ void stats_of_stored(float value, uint32_t bits, float pre_mult, float& acc, uint32_t& bad)
+{
+    constexpr uint32_t kExp = (AT == FT_F32) ? 0x7f800000u : (AT == FT_BF16 ? 0x7f80u : 0x7c00u);
+    const bool nf = (bits & kExp) == kExp;
+    const float x = value * pre_mult;
+    bad += nf ? 1u : 0u;
+    acc = __builtin_fmaf(nf ? 0.0f : x, nf ? 0.0f : x, acc);
+}
+
+template <int AT, int GT, bool ZERO, bool STATS>
+__device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, float scale, float pre_mult,
+                                                float (&sums)[4], uint32_t& bad)
+{
+    const f32x4 g4 = load_g4<GT, true>(g, i);
+    f32x4 a4;
+    if constexpr (AT == FT_F32) {
+        a4 = reinterpret_cast<const f32x4*>(acc)[i];
+    } else {
+        const u32x2 w = reinterpret_cast<const u32x2*>(acc)[i];
+        a4.x = half_to_float<AT>(w.x & 0xffffu);
+        a4.y = half_to_float<AT>(w.x >> 16);
+        a4.z = half_to_float<AT>(w.y & 0xffffu);
+        a4.w = half_to_float<AT>(w.y >> 16);
+    }
+    f32x4 r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float x = __builtin_fmaf(g4[k], scale, a4[k]);
+        asm volatile("" : "+v"(x));  // round to fp32 first; a narrowing store must see this value
+        r[k] = x;
+    }
+    if constexpr (AT == FT_F32) {
+        reinterpret_cast<f32x4*>(acc)[i] = r;
+        if constexpr (STATS) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float rk = r[k];  // a scalar copy: bit-casting the vector element itself reads lane 0
+                stats_of_stored<FT_F32>(rk, __builtin_bit_cast(uint32_t, rk), pre_mult, sums[k], bad);
+            }
+        }
+    } else {
+        u32x2 w;
+        w.x = pack2<AT>(r.x, r.y);
+        w.y = pack2<AT>(r.z, r.w);
+        reinterpret_cast<u32x2*>(acc)[i] = w;
+        if constexpr (STATS) {
+            const uint32_t b[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) stats_of_stored<AT>(half_to_float<AT>(b[k]), b[k], pre_mult, sums[k], bad);
+        }
+    }
+    if constexpr (ZERO) {
+        if constexpr (GT == FT_F32) {
+            const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            reinterpret_cast<f32x4*>(g)[i] = z;
+        } else {
+            const u32x2 z = {0u, 0u};
+            reinterpret_cast<u32x2*>(g)[i] = z;
+        }
+    }
+}
+
+// nvec = number of 4-element units. With STATS every block writes partials[blockIdx.x].
+template <int AT, int GT, bool ZERO, bool STATS, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void grad_accumulate_kernel(void* acc, void* g, uint64_t nvec, float scale,
+                                                                float pre_mult, StatsPartial* __restrict__ partials)
+{
+    float sums[4] = {0.f, 0.f, 0.f, 0.f};
+    uint32_t bad = 0;
+    const uint64_t stride = (uint64_t)gridDim.x * BLOCK;
+    for (uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x; i < nvec; i += stride)
+        accumulate_unit<AT, GT, ZERO, STATS>(acc, g, i, scale, pre_mult, sums, bad);
+    if constexpr (STATS) block_stats_epilogue<BLOCK>(sums, bad, partials);
+}
+
+// Elements outside the vector body, one by one, by a single thread; writes one more partial.
+template <int AT, int GT, bool ZERO, bool STATS>
+__global__ void grad_accumulate_edge_kernel(void* acc, void* g, uint64_t head, uint64_t tail_begin, uint64_t n,
+                                            float scale, float pre_mult, StatsPartial* partial)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    double s = 0.0;
+    uint64_t b = 0;
+    for (uint64_t i = 0; i < n; ++i) {
+        if (i == head) i = tail_begin;
+        if (i >= n) break;
+        float gi;
+        if constexpr (GT == FT_F32)
+            gi = reinterpret_cast<const float*>(g)[i];
+        else
+            gi = half_to_float<GT>(reinterpret_cast<const uint16_t*>(g)[i]);
+        float ai;
+        if constexpr (AT == FT_F32)
+            ai = reinterpret_cast<const float*>(acc)[i];
+        else
+            ai = half_to_float<AT>(reinterpret_cast<const uint16_t*>(acc)[i]);
+        float x = __builtin_fmaf(gi, scale, ai);
+        asm volatile("" : "+v"(x));
+        uint32_t bits;
+        float stored;
+        if constexpr (AT == FT_F32) {
+            reinterpret_cast<float*>(acc)[i] = x;
+            bits = __builtin_bit_cast(uint32_t, x);
+            stored = x;
+        } else {
+            bits = pack2<AT>(x, 0.0f) & 0xffffu;
+            reinterpret_cast<uint16_t*>(acc)[i] = (uint16_t)bits;
+            stored = half_to_float<AT>(bits);
+        }
+        if constexpr (STATS) {
+            float one = 0.f;
+            uint32_t nb = 0;
+            stats_of_stored<AT>(stored, bits, pre_mult, one, nb);
+            s += (double)one;
+            b += nb;
+        }
+        if constexpr (ZERO) {
+            if constexpr (GT == FT_F32)
+                reinterpret_cast<float*>(g)[i] = 0.0f;
+            else
+                reinterpret_cast<uint16_t*>(g)[i] = 0;
+        }
+    }
+    if constexpr (STATS) {
+        partial->sumsq = s;
+        partial->nonfinite = b;
     }
 }
 

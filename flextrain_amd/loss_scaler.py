@@ -196,6 +196,28 @@ class GradientGuard:
                 0 if self._fresh else 1, self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(grads.device)))
         self._fresh = False
 
+    def accumulate(self, acc: torch.Tensor, grads: torch.Tensor, scale: float = 1.0, zero_grads: bool = False,
+                   with_stats: bool = False, loss_scale: float = 1.0) -> None:
+        """``acc += scale * grads`` in one pass (one fused multiply-add per element, rounded to
+        ``acc``'s dtype), optionally clearing ``grads`` and -- ``with_stats`` -- gathering the
+        statistics of the new ``acc`` as ``add(acc, loss_scale)`` would, so that the last
+        accumulation of a step needs no separate statistics pass. Replaces the reference's
+        per-micro-batch ``gradacc_buffer += extra_grads`` and ``zero_`` pair
+        (``flextrain/memory/coordinator/optimizer.py:743,775-777``)."""
+        for name, t in (("acc", acc), ("grads", grads)):
+            if not t.is_cuda or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous GPU tensor")
+        if acc.numel() != grads.numel():
+            raise ValueError("acc and grads must have the same number of elements")
+        stats_ptr = self.stats_ptr if with_stats else None
+        with torch.cuda.device(acc.device):
+            _C.check("ft_grad_accumulate", self._lib.ft_grad_accumulate(
+                acc.data_ptr(), _C.dtype_code(acc.dtype), grads.data_ptr(), _C.dtype_code(grads.dtype), acc.numel(),
+                float(scale), int(bool(zero_grads)), float(1.0 / float(loss_scale)), stats_ptr,
+                0 if self._fresh else 1, self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(acc.device)))
+        if with_stats:
+            self._fresh = False
+
     def decide_async(self, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None) -> torch.Tensor:
         if self._fresh:
             raise RuntimeError("decide() before any add()")

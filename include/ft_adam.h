@@ -102,6 +102,19 @@ size_t ft_grad_stats_workspace_bytes(void);
 int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate,
                   void* workspace, size_t workspace_bytes, void* stream);
 
+/* ft_grad_accumulate: acc[i] = fma((float)g[i], scale, acc[i]) rounded to acc's type, in place;
+ * scale == 1 is the plain accumulation the reference performs after every micro-batch when
+ * gradients are accumulated in a wider type than they are produced in
+ * (flextrain/memory/coordinator/optimizer.py:771-777), other values fold in the averaging of
+ * flextrain/optimizer.py:250. zero_g != 0 also clears g, replacing the separate zeroing of the
+ * receive buffer (coordinator/optimizer.py:743). With stats_out != NULL the pass also produces the
+ * statistics ft_grad_stats would report for the new acc (pre-multiplied by stats_pre_mult), so
+ * the last accumulation of a step makes the separate statistics pass unnecessary.
+ * acc and g must start at the same element offset modulo 4 of their buffers. */
+int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                       float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
+                       size_t workspace_bytes, void* stream);
+
 /* ft_grad_control: turns statistics into the per-step decision, on the device:
  *   skip      = stats->nonfinite != 0
  *   norm      = sqrt(stats->sumsq)                                (double)
@@ -169,9 +182,11 @@ int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps);
 /* ---- launch tuning ------------------------------------------------------------------------
  * adam_waves_per_cu: how many 64-lane workgroups of the update kernel may be resident on one
  * compute unit (an occupancy throttle; 32 or more = no throttle). stats_blocks_per_cu: grid size
- * of the statistics kernel in 256-thread blocks per compute unit. A value <= 0 restores the
- * default. Affects speed only, never results. */
-int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu);
+ * of the statistics kernel in 256-thread blocks per compute unit. accumulate_waves_per_cu: grid
+ * size of the accumulation kernel in 64-lane workgroups per compute unit. A value <= 0 restores
+ * the default. Affects speed only, never results (the sum of squares may differ in its last bits
+ * with the grid, within the documented tolerance). */
+int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu, int accumulate_waves_per_cu);
 
 #ifdef __cplusplus
 }

@@ -79,6 +79,8 @@ def lib() -> ctypes.CDLL:
     L.ft_oracle_grad_stats.argtypes = [vp, i32, sz, f32, ctypes.POINTER(ctypes.c_uint64),
                                        ctypes.POINTER(ctypes.c_double), i32]
     L.ft_oracle_grad_stats.restype = i32
+    L.ft_oracle_grad_accumulate.argtypes = [vp, i32, vp, i32, sz, f32, i32]
+    L.ft_oracle_grad_accumulate.restype = i32
     L.ft_oracle_convert.argtypes = [vp, i32, vp, i32, sz]
     L.ft_oracle_convert.restype = None
     L.ft_oracle_best_isa.restype = i32
@@ -148,6 +150,16 @@ def grad_stats(g: np.ndarray, g_dtype: int, pre_mult: float = 1.0, threads: int 
     if rc != 0:
         raise RuntimeError("ft_oracle_grad_stats rejected its arguments")
     return int(bad.value), float(acc.value)
+
+
+def grad_accumulate(acc: np.ndarray, acc_dtype: int, g: np.ndarray, g_dtype: int, scale: float = 1.0,
+                    zero_g: bool = False) -> None:
+    """acc = round(fma(g, scale, acc)) in place (16-bit types as uint16 bit patterns)."""
+    n = acc.shape[0]
+    _check(acc, acc_dtype, n, "acc")
+    _check(g, g_dtype, n, "g")
+    if lib().ft_oracle_grad_accumulate(_ptr(acc), acc_dtype, _ptr(g), g_dtype, n, scale, int(bool(zero_g))) != 0:
+        raise RuntimeError("ft_oracle_grad_accumulate rejected its arguments")
 
 
 def convert(src: np.ndarray, src_dtype: int, dst_dtype: int) -> np.ndarray:

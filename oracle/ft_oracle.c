@@ -182,6 +182,35 @@ int ft_oracle_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult,
     return 0;
 }
 
+static float load_as_f32(const void* a, int dtype, size_t i)
+{
+    if (dtype == FT_ORACLE_F32) return ((const float*)a)[i];
+    if (dtype == FT_ORACLE_BF16) return fto_bf16_to_f32(((const uint16_t*)a)[i]);
+    return fto_f16_to_f32(((const uint16_t*)a)[i]);
+}
+
+int ft_oracle_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g)
+{
+    if (acc_dtype < 0 || acc_dtype > 2 || g_dtype < 0 || g_dtype > 2) return -1;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < n; ++i) {
+        const float x = fmaf(load_as_f32(g, g_dtype, i), scale, load_as_f32(acc, acc_dtype, i));
+        if (acc_dtype == FT_ORACLE_F32)
+            ((float*)acc)[i] = x;
+        else if (acc_dtype == FT_ORACLE_BF16)
+            ((uint16_t*)acc)[i] = fto_f32_to_bf16(x);
+        else
+            ((uint16_t*)acc)[i] = fto_f32_to_f16(x);
+        if (zero_g) {
+            if (g_dtype == FT_ORACLE_F32)
+                ((float*)g)[i] = 0.0f;
+            else
+                ((uint16_t*)g)[i] = 0;
+        }
+    }
+    return 0;
+}
+
 uint16_t ft_oracle_f32_to_f16(float x) { return fto_f32_to_f16(x); }
 uint16_t ft_oracle_f32_to_bf16(float x) { return fto_f32_to_bf16(x); }
 float ft_oracle_f16_to_f32(uint16_t h) { return fto_f16_to_f32(h); }

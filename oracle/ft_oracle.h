@@ -86,6 +86,13 @@ void ft_oracle_adam_trace(const ft_oracle_scalars* s, float grad_mult, float p, 
 int ft_oracle_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult,
                          uint64_t* out_nonfinite, double* out_sumsq, int threads);
 
+/* Gradient accumulation: acc[i] = round_to_acc_type(fmaf((float)g[i], scale, (float)acc[i])); with
+ * zero_g the gradient is cleared afterwards. No counterpart function in the reference; scale == 1
+ * is the `gradacc_buffer += extra_grads` of flextrain/memory/coordinator/optimizer.py:775-777
+ * (torch promotes the 16-bit operand exactly, then adds once). Pinned by numpy/torch adds and by
+ * exact rational arithmetic for scale != 1. */
+int ft_oracle_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g);
+
 /* Scalar conversions (software, no hardware conversion instructions). */
 uint16_t ft_oracle_f32_to_f16(float x);  /* IEEE binary16, round-to-nearest-even */
 uint16_t ft_oracle_f32_to_bf16(float x); /* bfloat16, round-to-nearest-even, NaN stays NaN */

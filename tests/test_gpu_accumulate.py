@@ -1,0 +1,97 @@
+"""GPU tests of the fused gradient accumulation pass (accumulate [+ scale] [+ clear source]
+[+ statistics]) against the oracle: bit-exact accumulators, exact inf/nan counts, norm within 1e-6."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from _util import CODE, NORM_RTOL, max_ulp_gpu, to_np
+
+pytestmark = pytest.mark.gpu
+
+N_7B_LAYER = 4 * 4096 ** 2 + 3 * 4096 * 11008 + 2 * 4096
+
+
+def _bits(t):
+    n = to_np(t)
+    return n.view(np.uint16) if n.dtype == np.float16 else n
+
+
+@pytest.mark.parametrize("acc_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("g_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("scale,zero", [(1.0, False), (0.25, True), (0.3, False)])
+def test_accumulate_matrix(cuda, oracle, acc_dtype, g_dtype, scale, zero):
+    from flextrain_amd.loss_scaler import GradientGuard
+    guard = GradientGuard(cuda)
+    gen = torch.Generator(device=cuda).manual_seed(3)
+    for n, offset in ((1, 0), (5, 3), (1000, 1), (4096, 0), (300_007, 2)):
+        A = torch.randn(n + offset + 8, device=cuda, generator=gen).to(acc_dtype)
+        G = (torch.randn(n + offset + 8, device=cuda, generator=gen) * 0.1).to(g_dtype)
+        a, g = A[offset:offset + n], G[offset:offset + n]
+        an, gn = _bits(a).copy(), _bits(g).copy()
+        oracle.grad_accumulate(an, CODE[acc_dtype], gn, CODE[g_dtype], scale=scale, zero_g=zero)
+        outside = (A[:offset].clone(), A[offset + n:].clone(), G[:offset].clone(), G[offset + n:].clone())
+        guard.accumulate(a, g, scale=scale, zero_grads=zero)
+        assert max_ulp_gpu(a, an) == 0, (n, offset)
+        assert np.array_equal(_bits(g), gn)  # cleared, or untouched
+        assert torch.equal(A[:offset], outside[0]) and torch.equal(A[offset + n:], outside[1])
+        assert torch.equal(G[:offset], outside[2]) and torch.equal(G[offset + n:], outside[3])
+
+
+def test_fused_statistics_equal_a_separate_pass(cuda, oracle):
+    from flextrain_amd.loss_scaler import GradientGuard
+    guard, check = GradientGuard(cuda), GradientGuard(cuda)
+    n, scale_loss = 1_000_003, 1024.0
+    acc = torch.zeros(n, device=cuda)
+    gen = torch.Generator(device=cuda).manual_seed(5)
+    micro = [(torch.randn(n, device=cuda, generator=gen) * 0.01 * scale_loss).to(torch.float16) for _ in range(4)]
+    micro[2][12345] = float("inf")
+    micro[3][0] = float("nan")
+    micro[3][n - 1] = float("-inf")
+    an = np.zeros(n, np.float32)
+    guard.begin()
+    for k, g in enumerate(micro):
+        last = k == len(micro) - 1
+        oracle.grad_accumulate(an, CODE[torch.float32], _bits(g).copy(), CODE[g.dtype], scale=0.25)
+        guard.accumulate(acc, g, scale=0.25, zero_grads=True, with_stats=last, loss_scale=scale_loss)
+        assert not g.any()
+    d = guard.decide(loss_scale=scale_loss, max_grad_norm=1.0)
+    assert max_ulp_gpu(acc, an) == 0
+    bad, sumsq = oracle.grad_stats(an, CODE[torch.float32], pre_mult=1.0 / scale_loss)
+    assert d.nonfinite == bad == 3 and d.overflow
+    assert abs(d.sumsq - sumsq) <= 2 * NORM_RTOL * sumsq
+    check.begin()
+    check.add(acc, loss_scale=scale_loss)
+    d2 = check.decide(loss_scale=scale_loss, max_grad_norm=1.0)
+    assert d2.nonfinite == d.nonfinite and abs(d2.sumsq - d.sumsq) <= 2 * NORM_RTOL * d.sumsq
+
+
+def test_mismatched_element_offsets_are_refused(cuda):
+    from flextrain_amd.loss_scaler import GradientGuard
+    guard = GradientGuard(cuda)
+    a, g = torch.zeros(1000, device=cuda), torch.zeros(1001, device=cuda, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="element offset"):
+        guard.accumulate(a, g[1:])
+    with pytest.raises(ValueError):
+        guard.accumulate(a, g)  # lengths differ
+
+
+def test_accumulate_llama7b_layer(cuda, oracle):
+    """Full-size: fp32 accumulator += bf16 gradients over the 7B-layer partition, with the
+    statistics of the result gathered in the same pass."""
+    from flextrain_amd.loss_scaler import GradientGuard
+    n = N_7B_LAYER
+    guard = GradientGuard(cuda)
+    gen = torch.Generator(device=cuda).manual_seed(9)
+    acc = torch.randn(n, device=cuda, generator=gen) * 1e-3
+    g = (torch.randn(n, device=cuda, generator=gen) * 1e-3).to(torch.bfloat16)
+    an, gn = to_np(acc).copy(), _bits(g).copy()
+    oracle.grad_accumulate(an, CODE[torch.float32], gn, CODE[torch.bfloat16], scale=1.0)
+    guard.begin()
+    guard.accumulate(acc, g, with_stats=True)
+    d = guard.decide()
+    assert max_ulp_gpu(acc, an) == 0
+    bad, sumsq = oracle.grad_stats(an, CODE[torch.float32])
+    assert d.nonfinite == bad == 0
+    assert abs(math.sqrt(d.sumsq) - math.sqrt(sumsq)) <= NORM_RTOL * math.sqrt(sumsq)

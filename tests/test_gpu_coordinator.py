@@ -76,3 +76,40 @@ def test_backward_pipeline_matches_oracle(cuda, oracle, offload):
     assert decay["step"] == 2 and plain["step"] == 2
     # the module's parameters are views of the flat unit buffers: they saw the update
     assert weights[0].data_ptr() == flat[0].data_ptr()
+
+
+def test_wider_accumulation_type(cuda, oracle):
+    """bf16 parameters and gradients, fp32 accumulation: each micro-batch is written into the extra
+    buffer and folded in by one fused pass; the step then consumes fp32 gradients."""
+    from flextrain_amd import FlexTrainAdam
+    from flextrain_amd.coordinator import FlexTrainOptsCoordinator
+    torch.manual_seed(1)
+    num_units, micro_batches, unit_numel = 3, 2, 1 << 18
+    flat = [(torch.randn(unit_numel, device=cuda) * 0.02).to(torch.bfloat16) for _ in range(num_units)]
+    params = [torch.nn.Parameter(f) for f in flat]
+    group = {"params": params, "weight_decay": 0.01}
+    opt = FlexTrainAdam([group], lr=1e-4, unit_parameter_map={u: _Unit([params[u]]) for u in range(num_units)},
+                        aligned_unit_numel=unit_numel, offload=False)
+    coord = FlexTrainOptsCoordinator()
+    coord.initialize(opt, flat, micro_batches, gradacc_dtype=torch.float32, offload=False)
+    state = [(to_np(flat[u].float()).copy(), np.zeros(unit_numel, np.float32), np.zeros(unit_numel, np.float32))
+             for u in range(num_units)]
+    opt.update_states()
+    acc = {u: np.zeros(unit_numel, np.float32) for u in range(num_units)}
+    for u in reversed(range(num_units)):
+        buf = coord.pre_unit_backward(u)
+        assert buf.dtype == torch.bfloat16
+        for mb in range(micro_batches):
+            g = (torch.randn(unit_numel, device=cuda) * 1e-3).to(torch.bfloat16)
+            buf.copy_(g)  # backward of one micro-batch writes its gradients
+            oracle.grad_accumulate(acc[u], CODE[torch.float32], to_np(g).copy(), CODE[torch.bfloat16])
+            coord.post_micro_batch_backward(u, mb)
+            assert not buf.any()  # cleared for the next micro-batch
+    coord.clear_backward_pipeline()
+    for u in range(num_units):
+        pn, mn, vn = state[u]
+        hn = np.zeros(unit_numel, np.uint16)
+        oracle.adam_step(pn, acc[u], mn, vn, step=1, lr=1e-4, weight_decay=0.01, half_out=hn, half_dtype=CODE[torch.bfloat16])
+        m, v = coord.unit_optimizer_states(u)
+        assert max_ulp(to_np(coord.unit_master_parameter(u)), pn) == 0 and max_ulp(to_np(m), mn) == 0
+        assert max_ulp(to_np(v), vn) == 0 and max_ulp(half_bits(flat[u]), hn, bf16=True) == 0

@@ -446,3 +446,30 @@ def test_loss_scale_traces(oracle):
     tr = oracle.loss_scale_trace([False] * 8, 4.0, scale_window=4)
     assert tr == [4.0, 4.0, 4.0, 4.0, 8.0, 8.0, 8.0, 8.0, 16.0]
     assert oracle.loss_scale_trace([True] * 4, 4.0, min_scale=1.0) == [4.0, 2.0, 1.0, 1.0, 1.0]
+
+
+def test_grad_accumulate_closed_forms(oracle):
+    """scale = 1: one add of the exactly widened gradient (numpy / torch); scale != 1: one fma,
+    checked in exact rationals; 16-bit accumulators: round-to-nearest-even of that fp32 value."""
+    rng = np.random.default_rng(11)
+    n = 5001
+    acc0 = rng.normal(0, 1, n).astype(np.float32)
+    g16 = (torch.randn(n) * 0.1).to(torch.bfloat16)
+    acc = acc0.copy()
+    gbits = g16.view(torch.int16).numpy().view(np.uint16).copy()
+    oracle.grad_accumulate(acc, oracle.F32, gbits, oracle.BF16)
+    assert np.array_equal(acc, acc0 + g16.float().numpy())
+    acc = acc0.copy()
+    scale = np.float32(0.3)
+    oracle.grad_accumulate(acc, oracle.F32, gbits, oracle.BF16, scale=float(scale), zero_g=True)
+    assert not gbits.any()
+    gf = g16.float().numpy()
+    for i in range(0, n, 50):
+        assert F(acc[i]) == fl32(F(gf[i]) * F(scale) + F(acc0[i]))
+    for code, dt in ((oracle.F16, torch.float16), (oracle.BF16, torch.bfloat16)):
+        a = (torch.randn(n) * 2).to(dt)
+        g = (torch.randn(n) * 0.5).to(torch.float16)
+        abits = a.view(torch.int16).numpy().view(np.uint16).copy()
+        oracle.grad_accumulate(abits, code, g.view(torch.int16).numpy().view(np.uint16).copy(), oracle.F16)
+        want = (a.float() + g.float()).to(dt).view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(abits, want)
