@@ -29,6 +29,7 @@ EXPORTS = {
                              c_void_p, c_void_p]),
     "ft_grad_stats_workspace_bytes": (c_size_t, []),
     "ft_grad_stats": (c_int, [c_void_p, c_int, c_size_t, c_float, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "ft_grad_accumulate_workspace_bytes": (c_size_t, [c_size_t]),
     "ft_grad_accumulate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_size_t, c_float, c_int, c_float, c_void_p, c_int,
                                    c_void_p, c_size_t, c_void_p]),
     "ft_grad_control": (c_int, [c_void_p, c_float, c_float, c_void_p, c_void_p]),
@@ -44,7 +45,7 @@ EXPORTS = {
     "ft_offload_wait": (c_int, [c_void_p]),
     "ft_offload_elapsed_ms": (c_int, [c_void_p, POINTER(c_float)]),
     "ft_link_bandwidth": (c_int, [c_size_t, c_int, c_int, POINTER(c_double)]),
-    "ft_set_launch_tuning": (c_int, [c_int, c_int, c_int]),
+    "ft_set_launch_tuning": (c_int, [c_int, c_int]),
 }
 
 

@@ -41,9 +41,6 @@
 #ifndef FT_STATS_UNROLL
 #define FT_STATS_UNROLL 4
 #endif
-#ifndef FT_ACCUM_WAVES_PER_CU
-#define FT_ACCUM_WAVES_PER_CU 12
-#endif
 #ifndef FT_STATS_BLOCKS_PER_CU
 #define FT_STATS_BLOCKS_PER_CU 4
 #endif
@@ -56,10 +53,10 @@ std::mutex g_mu;
 std::unordered_map<int, fth::AdamObject> g_adams;
 std::unordered_map<int, int> g_cu_count;      // device -> compute units
 std::unordered_map<int, void*> g_stats_ws;    // device -> library-owned statistics scratch
+std::unordered_map<int, size_t> g_stats_ws_bytes;
 int g_adam_waves_per_cu = FT_ADAM_WAVES_PER_CU;
 std::unordered_map<int, int> g_lds_per_cu;   // device -> bytes of LDS per compute unit
 int g_stats_blocks_per_cu = FT_STATS_BLOCKS_PER_CU;
-int g_accum_waves_per_cu = FT_ACCUM_WAVES_PER_CU;
 
 constexpr int kMaxStatsBlocks = 8192;
 
@@ -283,24 +280,28 @@ extern "C" size_t ft_grad_stats_workspace_bytes(void);
 
 namespace {
 
-// The caller's scratch if given (checked), else the per-device buffer the library owns.
-int resolve_stats_workspace(void* workspace, size_t workspace_bytes, ftk::StatsPartial** out)
+// The caller's scratch if given (checked against `need` bytes), else the per-device buffer the
+// library owns, grown when a call needs more than it holds (hipFree waits for the device, so work
+// still using the old buffer has finished before it goes away).
+int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need, ftk::StatsPartial** out)
 {
     ftk::StatsPartial* parts = static_cast<ftk::StatsPartial*>(workspace);
     if (parts) {
-        if (workspace_bytes < ft_grad_stats_workspace_bytes())
-            return fth::fail(FT_EINVAL, "workspace of %zu bytes is smaller than ft_grad_stats_workspace_bytes()",
-                             workspace_bytes);
+        if (workspace_bytes < need)
+            return fth::fail(FT_EINVAL, "workspace of %zu bytes is smaller than the %zu bytes this call needs",
+                             workspace_bytes, need);
         if (!aligned(parts, 16)) return fth::fail(FT_EALIGN, "workspace must be 16-byte aligned");
     } else {
         int dev = 0;
         FT_HIP(hipGetDevice(&dev));
         std::lock_guard<std::mutex> lk(g_mu);
         auto it = g_stats_ws.find(dev);
-        if (it == g_stats_ws.end()) {
+        if (it == g_stats_ws.end() || g_stats_ws_bytes[dev] < need) {
+            if (it != g_stats_ws.end()) FT_HIP(hipFree(it->second));
             void* w = nullptr;
-            FT_HIP(hipMalloc(&w, ft_grad_stats_workspace_bytes()));
+            FT_HIP(hipMalloc(&w, need));
             g_stats_ws[dev] = w;
+            g_stats_ws_bytes[dev] = need;
             parts = static_cast<ftk::StatsPartial*>(w);
         } else {
             parts = static_cast<ftk::StatsPartial*>(it->second);
@@ -310,55 +311,76 @@ int resolve_stats_workspace(void* workspace, size_t workspace_bytes, ftk::StatsP
     return FT_OK;
 }
 
+constexpr int kReduceBlocks = 256;  // second-level blocks of the accumulation pass's statistics
+
+// Wavefront partials of the accumulation pass live behind the fixed block-partial area.
+size_t accumulate_workspace_bytes(size_t n)
+{
+    const size_t waves = (n / 4 + 63) / 64;
+    return ft_grad_stats_workspace_bytes() + waves * sizeof(ftk::WavePartial);
+}
+
 template <int AT, int GT, bool ZERO, bool STATS>
 int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, float scale, float pre_mult,
-                      ftk::StatsPartial* parts, int blocks, hipStream_t stream)
+                      ftk::StatsPartial* parts, int* nparts, hipStream_t stream)
 {
     constexpr size_t asz = (AT == FT_F32) ? 4 : 2, gsz = (GT == FT_F32) ? 4 : 2;
+    int reduce_blocks = 0;
     if (nvec > 0) {
-        // Without statistics there are no per-block partials to bound, so the kernel runs like the
-        // update: one tile per wavefront-sized workgroup, residency throttled through dynamic LDS.
-        unsigned lds = 0;
-        if (!STATS) {
-            size_t b = (nvec + 63) / 64;
-            if (b > 0x7fffffffu) b = 0x7fffffffu;
-            blocks = static_cast<int>(b);
-            lds = fth::throttle_lds_bytes(4 * static_cast<unsigned>(asz + gsz));
-        }
-        hipLaunchKernelGGL((ftk::grad_accumulate_kernel<AT, GT, ZERO, STATS, 64>), dim3(blocks), dim3(64), lds, stream,
+        // Like the update: one tile per wavefront-sized workgroup, residency throttled through
+        // dynamic LDS so that the bytes in flight per compute unit stay at the tuned level.
+        size_t waves = (nvec + 63) / 64;
+        if (waves > 0x7fffffffu) waves = 0x7fffffffu;
+        ftk::WavePartial* wave_parts =
+            STATS ? reinterpret_cast<ftk::WavePartial*>(reinterpret_cast<char*>(parts) + ft_grad_stats_workspace_bytes())
+                  : nullptr;
+        // Measured: clearing the source adds a third of store traffic and the best residency
+        // drops by about that much, so the cleared variant is throttled as if it loaded a third more.
+        constexpr unsigned kLoadBytes = 4 * static_cast<unsigned>(asz + gsz);
+        constexpr unsigned kThrottleBytes = ZERO ? kLoadBytes + kLoadBytes / 3 : kLoadBytes;
+        hipLaunchKernelGGL((ftk::grad_accumulate_kernel<AT, GT, ZERO, STATS>), dim3(static_cast<unsigned>(waves)), dim3(64),
+                           fth::throttle_lds_bytes(kThrottleBytes), stream,
                            static_cast<void*>(static_cast<char*>(acc) + head * asz),
                            static_cast<void*>(static_cast<char*>(g) + head * gsz), static_cast<uint64_t>(nvec), scale,
-                           pre_mult, parts);
+                           pre_mult, wave_parts);
         FT_HIP(hipGetLastError());
+        if (STATS) {
+            reduce_blocks = waves < static_cast<size_t>(kReduceBlocks) ? static_cast<int>(waves) : kReduceBlocks;
+            const uint64_t per_block = (waves + reduce_blocks - 1) / reduce_blocks;
+            hipLaunchKernelGGL(ftk::reduce_wave_partials_kernel, dim3(reduce_blocks), dim3(256), 0, stream, wave_parts,
+                               static_cast<uint64_t>(waves), per_block, parts);
+            FT_HIP(hipGetLastError());
+        }
     }
     const size_t tail_begin = head + nvec * 4;
     if (STATS || head > 0 || tail_begin < n) {
         hipLaunchKernelGGL((ftk::grad_accumulate_edge_kernel<AT, GT, ZERO, STATS>), dim3(1), dim3(64), 0, stream, acc, g,
                            static_cast<uint64_t>(head), static_cast<uint64_t>(tail_begin), static_cast<uint64_t>(n),
-                           scale, pre_mult, parts + blocks);
+                           scale, pre_mult, parts + reduce_blocks);
         FT_HIP(hipGetLastError());
     }
+    *nparts = reduce_blocks + 1;
     return FT_OK;
 }
 
 template <int AT, int GT>
 int launch_accumulate_flags(bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec, float scale,
-                            float pre_mult, ftk::StatsPartial* parts, int blocks, hipStream_t stream)
+                            float pre_mult, ftk::StatsPartial* parts, int* nparts, hipStream_t stream)
 {
-    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
-    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
-    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
-    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
+    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
+    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
+    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
 }
 
 template <int AT>
 int launch_accumulate_g(int g_dtype, bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec,
-                        float scale, float pre_mult, ftk::StatsPartial* parts, int blocks, hipStream_t stream)
+                        float scale, float pre_mult, ftk::StatsPartial* parts, int* nparts, hipStream_t stream)
 {
     switch (g_dtype) {
-        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
-        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
-        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, blocks, stream);
+        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
+        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
+        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
     }
 }
 
@@ -421,6 +443,8 @@ int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, floa
 
 size_t ft_grad_stats_workspace_bytes(void) { return sizeof(ftk::StatsPartial) * kMaxStatsBlocks; }
 
+size_t ft_grad_accumulate_workspace_bytes(size_t n) { return accumulate_workspace_bytes(n); }
+
 int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate, void* workspace,
                   size_t workspace_bytes, void* stream_)
 {
@@ -432,7 +456,7 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
     if (n > 0 && !aligned(g, elem_size(g_dtype))) return fth::fail(FT_EALIGN, "g is not aligned to its element size");
 
     ftk::StatsPartial* parts = nullptr;
-    int wrc = resolve_stats_workspace(workspace, workspace_bytes, &parts);
+    int wrc = resolve_stats_workspace(workspace, workspace_bytes, ft_grad_stats_workspace_bytes(), &parts);
     if (wrc != FT_OK) return wrc;
 
     const size_t esz = elem_size(g_dtype);
@@ -510,27 +534,20 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
     }
     ftk::StatsPartial* parts = nullptr;
     if (stats) {
-        int wrc = resolve_stats_workspace(workspace, workspace_bytes, &parts);
+        int wrc = resolve_stats_workspace(workspace, workspace_bytes, accumulate_workspace_bytes(n), &parts);
         if (wrc != FT_OK) return wrc;
     }
-    int blocks = 0;
-    if (nvec > 0) {
-        size_t b = (nvec + 63) / 64;  // one wavefront per workgroup, a persistent grid of them
-        size_t cap = static_cast<size_t>(fth::cu_count()) * static_cast<size_t>(g_accum_waves_per_cu);
-        if (cap > static_cast<size_t>(kMaxStatsBlocks - 1)) cap = kMaxStatsBlocks - 1;
-        if (b > cap) b = cap;
-        blocks = static_cast<int>(b);
-    }
+    int nparts = 0;
     int rc;
     switch (acc_dtype) {
-        case FT_F32: rc = launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, blocks, stream); break;
-        case FT_F16: rc = launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, blocks, stream); break;
-        default: rc = launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, blocks, stream); break;
+        case FT_F32: rc = launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, &nparts, stream); break;
+        case FT_F16: rc = launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, &nparts, stream); break;
+        default: rc = launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, &nparts, stream); break;
     }
     if (rc != FT_OK) return rc;
     if (stats) {
-        // block partials [0, blocks) plus the edge kernel's one at index `blocks`
-        hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, blocks + 1,
+        // second-level partials plus the edge kernel's one
+        hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, nparts,
                            static_cast<const void*>(nullptr), static_cast<uint64_t>(0), static_cast<uint64_t>(0),
                            static_cast<uint64_t>(0), 1.0f, static_cast<ft_grad_stats_t*>(stats_out), stats_accumulate);
         FT_HIP(hipGetLastError());
@@ -550,10 +567,9 @@ int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ct
     return FT_OK;
 }
 
-int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu, int accumulate_waves_per_cu)
+int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu)
 {
     std::lock_guard<std::mutex> lk(g_mu);
-    g_accum_waves_per_cu = accumulate_waves_per_cu > 0 ? accumulate_waves_per_cu : FT_ACCUM_WAVES_PER_CU;
     g_adam_waves_per_cu = adam_waves_per_cu > 0 ? adam_waves_per_cu : FT_ADAM_WAVES_PER_CU;
     g_stats_blocks_per_cu = stats_blocks_per_cu > 0 ? stats_blocks_per_cu : FT_STATS_BLOCKS_PER_CU;
     return FT_OK;

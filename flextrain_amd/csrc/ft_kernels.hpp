@@ -482,17 +482,68 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
     }
 }
 
-// nvec = number of 4-element units. With STATS every block writes partials[blockIdx.x].
-template <int AT, int GT, bool ZERO, bool STATS, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void grad_accumulate_kernel(void* acc, void* g, uint64_t nvec, float scale,
-                                                                float pre_mult, StatsPartial* __restrict__ partials)
+// What one wavefront-sized workgroup of the accumulation pass reports: 8 bytes per 256 elements.
+struct WavePartial {
+    float sumsq;
+    uint32_t nonfinite;
+};
+
+// nvec = number of 4-element units; one 64-lane workgroup per 64 units (the loop only matters when
+// the grid had to be capped). With STATS every workgroup writes wave_partials[blockIdx.x].
+template <int AT, int GT, bool ZERO, bool STATS>
+__global__ __launch_bounds__(64) void grad_accumulate_kernel(void* acc, void* g, uint64_t nvec, float scale,
+                                                             float pre_mult, WavePartial* __restrict__ wave_partials)
 {
     float sums[4] = {0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    const uint64_t stride = (uint64_t)gridDim.x * BLOCK;
-    for (uint64_t i = (uint64_t)blockIdx.x * BLOCK + threadIdx.x; i < nvec; i += stride)
+    const uint64_t stride = (uint64_t)gridDim.x * 64;
+    for (uint64_t i = (uint64_t)blockIdx.x * 64 + threadIdx.x; i < nvec; i += stride)
         accumulate_unit<AT, GT, ZERO, STATS>(acc, g, i, scale, pre_mult, sums, bad);
-    if constexpr (STATS) block_stats_epilogue<BLOCK>(sums, bad, partials);
+    if constexpr (STATS) {
+        const float t = wave_sum((sums[0] + sums[1]) + (sums[2] + sums[3]));
+        const uint32_t tb = wave_sum_u32(bad);
+        if (threadIdx.x == 0) {
+            WavePartial w;
+            w.sumsq = t;
+            w.nonfinite = tb;
+            wave_partials[blockIdx.x] = w;
+        }
+    }
+}
+
+// Second level: block r adds the contiguous slice [r*per_block, (r+1)*per_block) of the wavefront
+// partials in fp64, lanes striding the slice, then a fixed tree; one StatsPartial per block. The
+// order of every addition is fixed by (count, gridDim), so the result is reproducible.
+__global__ __launch_bounds__(256) void reduce_wave_partials_kernel(const WavePartial* __restrict__ wave_partials,
+                                                                   uint64_t count, uint64_t per_block,
+                                                                   StatsPartial* __restrict__ partials)
+{
+    __shared__ double s_sum[256];
+    __shared__ uint64_t s_bad[256];
+    const uint64_t lo = (uint64_t)blockIdx.x * per_block;
+    uint64_t hi = lo + per_block;
+    if (hi > count) hi = count;
+    double s = 0.0;
+    uint64_t b = 0;
+    for (uint64_t i = lo + threadIdx.x; i < hi; i += 256) {
+        const WavePartial w = wave_partials[i];
+        s += (double)w.sumsq;
+        b += w.nonfinite;
+    }
+    s_sum[threadIdx.x] = s;
+    s_bad[threadIdx.x] = b;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
+            s_bad[threadIdx.x] += s_bad[threadIdx.x + w];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        partials[blockIdx.x].sumsq = s_sum[0];
+        partials[blockIdx.x].nonfinite = s_bad[0];
+    }
 }
 
 // Elements outside the vector body, one by one, by a single thread; writes one more partial.

@@ -210,6 +210,11 @@ class GradientGuard:
         if acc.numel() != grads.numel():
             raise ValueError("acc and grads must have the same number of elements")
         stats_ptr = self.stats_ptr if with_stats else None
+        if with_stats:
+            need = int(self._lib.ft_grad_accumulate_workspace_bytes(acc.numel()))
+            if need > self._ws_bytes:  # grows with the largest buffer seen (8 bytes per 256 elements)
+                self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+                self._ws_bytes = need
         with torch.cuda.device(acc.device):
             _C.check("ft_grad_accumulate", self._lib.ft_grad_accumulate(
                 acc.data_ptr(), _C.dtype_code(acc.dtype), grads.data_ptr(), _C.dtype_code(grads.dtype), acc.numel(),

@@ -110,7 +110,10 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
  * receive buffer (coordinator/optimizer.py:743). With stats_out != NULL the pass also produces the
  * statistics ft_grad_stats would report for the new acc (pre-multiplied by stats_pre_mult), so
  * the last accumulation of a step makes the separate statistics pass unnecessary.
- * acc and g must start at the same element offset modulo 4 of their buffers. */
+ * acc and g must start at the same element offset modulo 4 of their buffers. With statistics the
+ * workspace must hold ft_grad_accumulate_workspace_bytes(n) bytes (8 bytes per 256 elements on
+ * top of the fixed part), or be NULL for the library's own buffer. */
+size_t ft_grad_accumulate_workspace_bytes(size_t n);
 int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
                        float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
                        size_t workspace_bytes, void* stream);
@@ -180,13 +183,14 @@ int ft_offload_elapsed_ms(void* handle, float* out_ms);
 int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps);
 
 /* ---- launch tuning ------------------------------------------------------------------------
- * adam_waves_per_cu: how many 64-lane workgroups of the update kernel may be resident on one
- * compute unit (an occupancy throttle; 32 or more = no throttle). stats_blocks_per_cu: grid size
- * of the statistics kernel in 256-thread blocks per compute unit. accumulate_waves_per_cu: grid
- * size of the accumulation kernel in 64-lane workgroups per compute unit. A value <= 0 restores
- * the default. Affects speed only, never results (the sum of squares may differ in its last bits
- * with the grid, within the documented tolerance). */
-int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu, int accumulate_waves_per_cu);
+ * adam_waves_per_cu: how many 64-lane workgroups of the update kernel (16-bit gradients: 56 bytes
+ * of loads in flight per lane) may be resident on one compute unit; kernels with fewer bytes per
+ * lane (fp32 gradients more, the accumulation pass fewer) are scaled to the same bytes in flight.
+ * 32 or more = no throttle. stats_blocks_per_cu: grid size of the statistics kernel in 256-thread
+ * blocks per compute unit (this one changes the order of the fp64 additions, so the sum of
+ * squares may move in its last bits, within the documented tolerance). A value <= 0 restores the
+ * default. Otherwise speed only, never results. */
+int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu);
 
 #ifdef __cplusplus
 }
