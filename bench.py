@@ -52,17 +52,29 @@ def make_inputs(torch, n, g_dtype, g_std, device, scale=1.0):
     return p, g, m, v, h
 
 
-def cpu_baseline(n, budget_s=20.0):
-    """Times the reference CPU Adam (its own C++ compiled into oracle/_ref when present, else this
-    repository's restatement) on host buffers of the workload's size: fp32 gradients and an fp16
-    copy-out, the only form the reference supports. 1 warm-up call, then timed calls until the
-    budget is used (at least 3, at most 20); 20-80 percentile mean, as flextrain/auto_config.py
-    does for its own optimizer probe."""
+def _host_description():
+    """CPU model, logical CPUs and NUMA nodes of the machine the CPU baseline runs on."""
+    import glob
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cpu_model": model, "logical_cpus": os.cpu_count(), "numa_nodes": len(glob.glob("/sys/devices/system/node/node[0-9]*")) or 1}
+
+
+def _time_cpu_adam(n, budget_s):
+    """1 warm-up call, then timed calls until the budget is used (at least 3, at most 20) of the
+    reference CPU Adam with fp32 gradients and an fp16 copy-out on n elements in host memory.
+    Returns (seconds per call as a 20-80 percentile mean, number of timed calls, kind, flavour)."""
     import numpy as np
     import torch
 
     import oracle
-    threads = oracle.max_threads()
     ref = oracle.reference_module()
     tp = torch.randn(n) * 0.02
     tg = torch.randn(n) * 1e-3
@@ -91,14 +103,31 @@ def cpu_baseline(n, budget_s=20.0):
         times.append(time.perf_counter() - t0)
     if ref is not None:
         ref.destroy_adam(oid)
-    sec = percentile_mean(times)
-    return {
+    flavour = getattr(ref, "flavour", f"libftoracle isa={oracle.best_isa()}")
+    return percentile_mean(times), len(times), kind, flavour
+
+
+def cpu_baseline(n, budget_s=14.0):
+    """Times the reference CPU Adam (its own C++ compiled into oracle/_ref when present, else this
+    repository's restatement) on host buffers of the workload's size: fp32 gradients and an fp16
+    copy-out, the only form the reference supports; 20-80 percentile mean of the timed calls, as
+    flextrain/auto_config.py:281-317 does for its own optimizer probe. The same is then timed on
+    the block size that probe itself uses (2**28 elements) and reported beside it."""
+    import oracle
+    threads = oracle.max_threads()
+    sec, calls, kind, flavour = _time_cpu_adam(n, budget_s)
+    out = {
         "value": n / sec, "unit": "elements/s", "cores": threads, "kind": kind,
-        "sample": f"{len(times)} timed calls (1 warm-up) of the CPU Adam with fp16 copy-out on {n} fp32 elements "
+        "sample": f"{calls} timed calls (1 warm-up) of the CPU Adam with fp16 copy-out on {n} fp32 elements "
                   f"in host memory, {threads} OpenMP threads, 20-80 percentile mean",
-        "ms_per_call": sec * 1e3, "host_gbps": n * 30 / sec / 1e9,
-        "flavour": getattr(ref, "flavour", f"libftoracle isa={oracle.best_isa()}"),
+        "ms_per_call": sec * 1e3, "host_gbps": n * 30 / sec / 1e9, "flavour": flavour,
+        "host": _host_description(),
     }
+    block = 1 << 28
+    bsec, bcalls, _, _ = _time_cpu_adam(block, budget_s * 0.4)
+    out["reference_probe_block"] = {"elements": block, "value": block / bsec, "unit": "elements/s",
+                                    "ms_per_call": bsec * 1e3, "timed_calls": bcalls}
+    return out
 
 
 def bench_offload(args, torch, dev) -> int:

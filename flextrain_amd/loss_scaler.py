@@ -235,6 +235,10 @@ class GradientGuard:
 
     def decide(self, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None) -> GuardDecision:
         self.decide_async(loss_scale, max_grad_norm)
+        return self.read()
+
+    def read(self) -> GuardDecision:
+        """The decision last taken by ``decide_async`` (reads 32 bytes back; waits for the stream)."""
         host = self._buf.cpu()  # synchronises with the current stream
         nonfinite = int(host[0:1].view(torch.int64).item())
         sumsq = float(host[1].item())

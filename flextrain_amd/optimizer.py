@@ -56,14 +56,49 @@ class FlexTrainCPUOptimizer(ABC):
         pass
 
     @torch.no_grad()
-    def step(self, step_contexts: Union[StepContext, List[StepContext]], **extensions):
+    def step(self, step_contexts: Union[StepContext, List[StepContext]], *, loss_scale: float = 1.0,
+             max_grad_norm: Optional[float] = None, check_overflow: bool = False, **extensions):
         """Steps every context; contexts without gradient elements are skipped
         (reference ``flextrain/optimizer.py:44-69``).
 
-        ``extensions`` (``grad_mult``, ``control``) are forwarded to ``_step`` unchanged.
+        Keyword-only additions, whose defaults give the reference's behaviour:
+          loss_scale: the gradients were produced from ``loss * loss_scale``; the update divides
+            them by it (one fp32 multiply by ``1/loss_scale``) on the fly.
+          check_overflow: look for inf/nan in the gradients of ALL the given contexts first; if any
+            is found no context is stepped (parameters and states keep their bits).
+          max_grad_norm: clip the L2 norm of the unscaled gradients of all the given contexts
+            together to this value.
+        With ``check_overflow`` or ``max_grad_norm`` the decision is taken on the device and the
+        call returns a ``GuardDecision`` (a 32-byte read-back after the update is enqueued; the
+        caller advances ``group["step"]`` and the loss scale from it); otherwise it returns None.
+        Gradients must then be GPU tensors. Other ``extensions`` (``grad_mult``, ``control``,
+        ``blocking``) are forwarded to ``_step`` unchanged.
         """
         if isinstance(step_contexts, StepContext):
             step_contexts = [step_contexts]
+        guard = None
+        if check_overflow or max_grad_norm is not None:
+            if "control" in extensions or "grad_mult" in extensions:
+                raise ValueError("check_overflow / max_grad_norm compute the control record themselves; "
+                                 "do not pass control or grad_mult as well")
+            live = [ctx.gradient for ctx in step_contexts if ctx.gradient.numel()]
+            if live:
+                from .loss_scaler import GradientGuard  # local import: keeps module load light
+                guard = self.__dict__.get("_step_guard")
+                if guard is None or guard.device != live[0].device:
+                    guard = self._step_guard = GradientGuard(live[0].device)
+                guard.begin()
+                for g in live:
+                    guard.add(g, loss_scale=loss_scale)
+                extensions["control"] = guard.decide_async(loss_scale=loss_scale, max_grad_norm=max_grad_norm)
+        elif loss_scale != 1.0:
+            if "control" in extensions:
+                raise ValueError("loss_scale is already part of the control record passed in")
+            extensions["grad_mult"] = float(extensions.get("grad_mult", 1.0)) * float(1.0 / float(loss_scale))
+        self._step_all(step_contexts, extensions)
+        return guard.read() if guard is not None else None
+
+    def _step_all(self, step_contexts: List[StepContext], extensions) -> None:
         for ctx in step_contexts:
             if not ctx.gradient.numel():
                 continue

@@ -194,3 +194,60 @@ def test_config4_clip_llama70b_layer(cuda, oracle):
     eng._step({"step": 1000}, h, p, g, m, v, control=guard.control)
     hn = _apply_oracle(oracle, pn, mn, vn, g, 1000, d.grad_mult, torch.bfloat16)
     _check_state("cfg4", p, m, v, h, pn, mn, vn, hn)
+
+
+def test_step_keywords_check_overflow_and_clip(cuda, oracle):
+    """`FlexTrainCPUOptimizer.step(contexts, loss_scale=, max_grad_norm=, check_overflow=)`: the
+    statistics cover the gradients of all contexts together, an inf in one context stops every
+    context, and an applied step equals the oracle with the returned multiplier."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.param_group import StepContext
+    eng = FlexTrainCPUAdam(**HP)
+    gen = torch.Generator(device=cuda).manual_seed(21)
+    scale = 256.0
+    sizes = (70_001, 0, 12_345)
+    ctxs, host = [], []
+    for n in sizes:
+        p = torch.randn(n, device=cuda, generator=gen) * 0.02
+        m = torch.randn(n, device=cuda, generator=gen) * 1e-4
+        v = torch.rand(n, device=cuda, generator=gen) * 1e-6
+        g = (torch.randn(n, device=cuda, generator=gen) * (5e-2 * scale)).to(torch.float16)
+        h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+        ctxs.append(StepContext({"step": 1}, h, p, g, [m, v]))
+        host.append([to_np(p).copy(), to_np(m).copy(), to_np(v).copy()])
+
+    # plain reference behaviour: no keywords, nothing returned
+    assert eng.step([]) is None
+
+    # overflow in the LAST context: nothing moves anywhere
+    ctxs[2].gradient[17] = float("inf")
+    before = [[t.clone() for t in (c.full_parameter, *c.optimizer_states, c.half_parameter)] for c in ctxs]
+    d = eng.step(ctxs, loss_scale=scale, check_overflow=True)
+    assert d.overflow and d.nonfinite == 1
+    for c, was in zip(ctxs, before):
+        for now, old in zip((c.full_parameter, *c.optimizer_states, c.half_parameter), was):
+            assert torch.equal(now, old)
+
+    # repaired gradient: the step is applied with the clip of the joint norm
+    ctxs[2].gradient[17] = 0.0
+    d = eng.step(ctxs, loss_scale=scale, max_grad_norm=1.0, check_overflow=True)
+    assert not d.overflow
+    sumsq = sum(oracle.grad_stats(_bits(c.gradient), CODE[torch.float16], pre_mult=1.0 / scale)[1]
+                for c in ctxs if c.gradient.numel())
+    assert abs(d.grad_norm - math.sqrt(sumsq)) <= 2 * NORM_RTOL * math.sqrt(sumsq)
+    assert d.clip_coef < 0.1  # norm ~ 0.05 * sqrt(82k) >> 1
+    for c, (pn, mn, vn) in zip(ctxs, host):
+        if not c.gradient.numel():
+            continue
+        hn = _apply_oracle(oracle, pn, mn, vn, c.gradient, 1, d.grad_mult, torch.bfloat16)
+        _check_state("step keywords", c.full_parameter, c.optimizer_states[0], c.optimizer_states[1],
+                     c.half_parameter, pn, mn, vn, hn)
+
+    # loss_scale alone: a host-side multiplier, no statistics, nothing returned
+    pn, mn, vn = host[0]
+    assert eng.step(ctxs[0], loss_scale=scale) is None
+    hn = _apply_oracle(oracle, pn, mn, vn, ctxs[0].gradient, 1, 1.0 / scale, torch.bfloat16)
+    _check_state("loss_scale only", ctxs[0].full_parameter, *ctxs[0].optimizer_states, ctxs[0].half_parameter, pn, mn, vn, hn)
+
+    with pytest.raises(ValueError):
+        eng.step(ctxs, check_overflow=True, grad_mult=0.5)
