@@ -28,7 +28,7 @@ N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 8
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
 # profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_703_000, "cfg3": 5_666_710_000, "cfg4": None}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_703_000, "cfg3": 5_666_710_000, "cfg4": 23_958_258_000, "accumulate": 2_453_892_000}
 
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
 
@@ -245,6 +245,12 @@ def bench_accumulate(args, torch, dev) -> int:
     guard = GradientGuard(dev)
     acc = torch.zeros(n, device=dev)
     g = (torch.randn(n, device=dev) * 1e-3).to(torch.bfloat16)
+    if args.calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
+        scratch = torch.empty_like(acc)
+        for _ in range(3):
+            scratch.copy_(acc)
+        torch.cuda.synchronize()
+        del scratch
     variants = {
         "accumulate": dict(zero_grads=False, with_stats=False, bytes=10),
         "accumulate+clear": dict(zero_grads=True, with_stats=False, bytes=12),
@@ -278,7 +284,8 @@ def bench_accumulate(args, torch, dev) -> int:
         "config": {"workload": "accumulate: fp32 accumulator += bf16 gradient on the 7B-layer partition, source cleared, "
                                "statistics of the result in the same pass", "elements": n},
         "roofline": {"bound": "hbm", "kernel": "grad_accumulate_kernel", "achieved": main["achieved_gbps"],
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": main["achieved_gbps"] / HBM_PEAK_GBPS, "traffic": None,
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": main["achieved_gbps"] / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES["accumulate"],
                      "algorithmic_bytes_per_launch": n * 12, "kernel_ms_avg": main["ms_avg"]},
         "variants": results,
     }), flush=True)
