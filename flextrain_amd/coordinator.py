@@ -212,6 +212,41 @@ class FlexTrainOptsCoordinator:
         else:
             torch.cuda.current_stream().synchronize()
 
+    # ---- state files ---------------------------------------------------------------------------
+    def save_optimizer_states(self, directory: str, *, rank: int = 0, checkpoint_interval: int = 1,
+                              fsync: bool = False) -> List[str]:
+        """Writes every unit's ``[master | exp_avg | exp_avg_sq]`` block as the reference's
+        backward-share swap file ``rank{r}_OPTS_layer{i}.swp.1`` (this coordinator has no forward
+        share, so there is no ``.0`` file, as for any empty share in the reference). Waits for the
+        steps in flight first. Returns the paths."""
+        from .state_files import BACKWARD_SHARE, write_unit_opts
+        self.synchronize()
+        paths = []
+        for u in range(self._num_units):
+            blocks = self._unit_opts[u] if self._offload else [b.cpu() for b in self._unit_opts[u]]
+            paths.append(write_unit_opts(directory, u, blocks, share=BACKWARD_SHARE, rank=rank,
+                                         checkpoint_interval=checkpoint_interval, fsync=fsync))
+        return paths
+
+    def load_optimizer_states(self, directory: str, *, rank: int = 0, checkpoint_interval: int = 1) -> None:
+        """Reads the files ``save_optimizer_states`` wrote back into the units' blocks and rounds
+        the master parameters into the units' low-precision parameters (what the update's copy-out
+        would have left there). Group step counters are the caller's to restore."""
+        from .state_files import BACKWARD_SHARE, read_unit_opts
+        self.synchronize()
+        for u in range(self._num_units):
+            if self._offload:
+                read_unit_opts(directory, u, self._unit_opts[u], share=BACKWARD_SHARE, rank=rank,
+                               checkpoint_interval=checkpoint_interval)
+            else:
+                staging = [torch.empty(b.shape, dtype=b.dtype) for b in self._unit_opts[u]]
+                read_unit_opts(directory, u, staging, share=BACKWARD_SHARE, rank=rank,
+                               checkpoint_interval=checkpoint_interval)
+                for dst, src in zip(self._unit_opts[u], staging):
+                    dst.copy_(src)
+            self._unit_half_parameters[u].copy_(self._unit_opts[u][0])
+        torch.cuda.current_stream().synchronize()
+
 
 _OPTS_COORDINATOR = FlexTrainOptsCoordinator()
 
