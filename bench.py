@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the optimizer-step hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5|pipeline|accumulate] [--no-cpu-baseline]
 
 A "step" is one fused AdamW update over one synthetic partition that is already resident in HBM.
 Default workload: the Llama-7B decoder-layer partition (202,383,360 elements, bf16 gradients,
