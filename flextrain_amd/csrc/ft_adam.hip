@@ -334,12 +334,8 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
         ftk::WavePartial* wave_parts =
             STATS ? reinterpret_cast<ftk::WavePartial*>(reinterpret_cast<char*>(parts) + ft_grad_stats_workspace_bytes())
                   : nullptr;
-        // Measured: clearing the source adds a third of store traffic and the best residency
-        // drops by about that much, so the cleared variant is throttled as if it loaded a third more.
-        constexpr unsigned kLoadBytes = 4 * static_cast<unsigned>(asz + gsz);
-        constexpr unsigned kThrottleBytes = ZERO ? kLoadBytes + kLoadBytes / 3 : kLoadBytes;
         hipLaunchKernelGGL((ftk::grad_accumulate_kernel<AT, GT, ZERO, STATS>), dim3(static_cast<unsigned>(waves)), dim3(64),
-                           fth::throttle_lds_bytes(kThrottleBytes), stream,
+                           fth::throttle_lds_bytes(4 * static_cast<unsigned>(asz + gsz)), stream,
                            static_cast<void*>(static_cast<char*>(acc) + head * asz),
                            static_cast<void*>(static_cast<char*>(g) + head * gsz), static_cast<uint64_t>(nvec), scale,
                            pre_mult, wave_parts);

@@ -435,10 +435,11 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
 {
     const f32x4 g4 = load_g4<GT, true>(g, i);
     f32x4 a4;
+    // Streaming accesses throughout: every buffer is far larger than the caches and is touched once.
     if constexpr (AT == FT_F32) {
-        a4 = reinterpret_cast<const f32x4*>(acc)[i];
+        a4 = ld<true>(reinterpret_cast<const f32x4*>(acc) + i);
     } else {
-        const u32x2 w = reinterpret_cast<const u32x2*>(acc)[i];
+        const u32x2 w = ld<true>(reinterpret_cast<const u32x2*>(acc) + i);
         a4.x = half_to_float<AT>(w.x & 0xffffu);
         a4.y = half_to_float<AT>(w.x >> 16);
         a4.z = half_to_float<AT>(w.y & 0xffffu);
@@ -452,7 +453,7 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
         r[k] = x;
     }
     if constexpr (AT == FT_F32) {
-        reinterpret_cast<f32x4*>(acc)[i] = r;
+        st<true>(reinterpret_cast<f32x4*>(acc) + i, r);
         if constexpr (STATS) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -464,7 +465,7 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
         u32x2 w;
         w.x = pack2<AT>(r.x, r.y);
         w.y = pack2<AT>(r.z, r.w);
-        reinterpret_cast<u32x2*>(acc)[i] = w;
+        st<true>(reinterpret_cast<u32x2*>(acc) + i, w);
         if constexpr (STATS) {
             const uint32_t b[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
 #pragma unroll
@@ -474,10 +475,10 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
     if constexpr (ZERO) {
         if constexpr (GT == FT_F32) {
             const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            reinterpret_cast<f32x4*>(g)[i] = z;
+            st<true>(reinterpret_cast<f32x4*>(g) + i, z);
         } else {
             const u32x2 z = {0u, 0u};
-            reinterpret_cast<u32x2*>(g)[i] = z;
+            st<true>(reinterpret_cast<u32x2*>(g) + i, z);
         }
     }
 }
