@@ -295,43 +295,47 @@ __device__ __forceinline__ void stats_accumulate(u32x4 w, float pre_mult, float 
     }
 }
 
-// Block-level end of a statistics pass: per-lane fp32 sums and counts -> one fp64 partial per block.
+// Block-level end of a statistics pass: per-lane fp64 sums and counts -> one partial per block,
+// added in a fixed tree order through LDS.
 template <int BLOCK>
-__device__ __forceinline__ void block_stats_epilogue(const float (&acc)[4], uint32_t bad, StatsPartial* __restrict__ partials)
+__device__ __forceinline__ void block_stats_epilogue(double lane_sum, uint32_t bad, StatsPartial* __restrict__ partials)
 {
-    const float t = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+    __shared__ double s_sum[BLOCK];
+    __shared__ uint32_t s_bad[BLOCK / kWave];
     const uint32_t tb = wave_sum_u32(bad);
-
-    constexpr int kWaves = BLOCK / kWave;
-    __shared__ float s_sum[kWaves];
-    __shared__ uint32_t s_bad[kWaves];
-    const int wave = threadIdx.x / kWave;
-    if ((threadIdx.x & (kWave - 1)) == 0) {
-        s_sum[wave] = t;
-        s_bad[wave] = tb;
-    }
+    s_sum[threadIdx.x] = lane_sum;
+    if ((threadIdx.x & (kWave - 1)) == 0) s_bad[threadIdx.x / kWave] = tb;
     __syncthreads();
+#pragma unroll
+    for (int w = BLOCK / 2; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
+        __syncthreads();
+    }
     if (threadIdx.x == 0) {
-        double s = 0.0;
         uint64_t b = 0;
 #pragma unroll
-        for (int k = 0; k < kWaves; ++k) {
-            s += (double)s_sum[k];
-            b += s_bad[k];
-        }
-        partials[blockIdx.x].sumsq = s;
+        for (int k = 0; k < BLOCK / kWave; ++k) b += s_bad[k];
+        partials[blockIdx.x].sumsq = s_sum[0];
         partials[blockIdx.x].nonfinite = b;
     }
 }
 
 // Stage 1: every block writes one StatsPartial. nvec = number of 16-byte units; the caller
 // handles the elements outside [0, nvec*per_unit) in grad_stats_final_kernel.
+// A lane adds squares in four fp32 accumulators and empties them into an fp64 sum every
+// kStatsFlushTiles tiles, so that no fp32 sum ever holds more than a few hundred terms however
+// many elements the call covers (with fp32 sums over the whole call the norm of 4e9 elements was
+// off by 3e-6).
+constexpr int kStatsFlushTiles = 16;
+
 template <int GT, int BLOCK, int UNROLL>
 __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restrict__ g, uint64_t nvec,
                                                            float pre_mult, StatsPartial* __restrict__ partials)
 {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    double lane_sum = 0.0;
     uint32_t bad = 0;
+    int pending = 0;
     constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -349,8 +353,14 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
                 stats_accumulate<GT>(g[i], pre_mult, acc, bad);
             }
         }
+        if (++pending == kStatsFlushTiles) {
+            lane_sum += ((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3]);
+            acc[0] = acc[1] = acc[2] = acc[3] = 0.f;
+            pending = 0;
+        }
     }
-    block_stats_epilogue<BLOCK>(acc, bad, partials);
+    lane_sum += ((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3]);
+    block_stats_epilogue<BLOCK>(lane_sum, bad, partials);
 }
 
 // Stage 2 (one block of 256): adds the block partials in a fixed tree order, then the up to
