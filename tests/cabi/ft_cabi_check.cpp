@@ -1,0 +1,251 @@
+// ft_cabi_check -- exercises libftadam.so through its C ABI alone, the way a binding in another
+// language would: HIP runtime for memory and a stream, plain pointers and sizes into the library,
+// no Python and no torch. Every result is compared bit for bit with the CPU checker
+// (libftoracle.so), which is test infrastructure and linked only into this test program.
+//
+// Prints one line per check and exits 0 when all passed. Needs a GPU.
+#include <hip/hip_runtime_api.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "ft_adam.h"
+#include "ft_oracle.h"
+
+namespace {
+
+int g_failures = 0;
+
+void check(bool ok, const char* what)
+{
+    std::printf("%s  %s\n", ok ? "ok  " : "FAIL", what);
+    std::fflush(stdout);
+    if (!ok) ++g_failures;
+}
+
+#define HIP_OK(expr)                                                                       \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            std::printf("FAIL  %s: %s\n", #expr, hipGetErrorString(e_));                   \
+            std::exit(2);                                                                  \
+        }                                                                                  \
+    } while (0)
+
+#define FT_OK_OR_DIE(expr)                                                                 \
+    do {                                                                                   \
+        int rc_ = (expr);                                                                  \
+        if (rc_ != FT_OK) {                                                                \
+            std::printf("FAIL  %s -> %d: %s\n", #expr, rc_, ft_last_error());              \
+            std::exit(2);                                                                  \
+        }                                                                                  \
+    } while (0)
+
+// splitmix64 -> uniform in (0, 1)
+struct Rng {
+    uint64_t s;
+    double uniform()
+    {
+        uint64_t z = (s += 0x9e3779b97f4a7c15ull);
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+        z ^= z >> 31;
+        return ((z >> 11) + 0.5) * (1.0 / 9007199254740992.0);
+    }
+    float normal(float std) { return std * (float)(std::sqrt(-2.0 * std::log(uniform())) * std::cos(6.283185307179586 * uniform())); }
+};
+
+template <typename T>
+T* dev_copy(const std::vector<T>& h)
+{
+    T* d = nullptr;
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&d), h.size() * sizeof(T) + 16));
+    HIP_OK(hipMemcpy(d, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice));
+    return d;
+}
+
+template <typename T>
+bool same_bits(const T* dev, const std::vector<T>& want)
+{
+    std::vector<T> got(want.size());
+    HIP_OK(hipMemcpy(got.data(), dev, want.size() * sizeof(T), hipMemcpyDeviceToHost));
+    return std::memcmp(got.data(), want.data(), want.size() * sizeof(T)) == 0;
+}
+
+const float LR = 1e-4f, B1 = 0.9f, B2 = 0.999f, EPS = 1e-8f, WD = 0.01f;
+
+void resident_mixed_precision_step(hipStream_t stream)
+{
+    const size_t n = 1000003;  // odd: head/tail paths
+    const float loss_scale = 1024.f;
+    const uint64_t t = 3;
+    Rng rng{42};
+    std::vector<float> p(n), m(n), v(n);
+    std::vector<uint16_t> g(n), h(n, 0);
+    for (size_t i = 0; i < n; ++i) {
+        p[i] = rng.normal(0.02f);
+        m[i] = rng.normal(1e-4f);
+        v[i] = (float)(rng.uniform() * 1e-6);
+        g[i] = ft_oracle_f32_to_f16(rng.normal(5e-3f) * loss_scale);
+    }
+    float *dp = dev_copy(p), *dm = dev_copy(m), *dv = dev_copy(v);
+    uint16_t *dg = dev_copy(g), *dh = dev_copy(h);
+    void* ws = nullptr;
+    char* rec = nullptr;  // ft_grad_stats_t followed by ft_step_control_t
+    HIP_OK(hipMalloc(&ws, ft_grad_stats_workspace_bytes()));
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&rec), 32));
+
+    FT_OK_OR_DIE(ft_adam_create(7, LR, B1, B2, EPS, WD, 1, 0));
+    FT_OK_OR_DIE(ft_grad_stats(dg, FT_F16, n, 1.f / loss_scale, rec, 0, ws, ft_grad_stats_workspace_bytes(), stream));
+    FT_OK_OR_DIE(ft_grad_control(rec, 1.f / loss_scale, 1.0f, rec + 16, stream));
+    FT_OK_OR_DIE(ft_adam_step(7, t, LR, B1, B2, EPS, WD, 1, 1.0f, dp, dg, FT_F16, dm, dv, dh, FT_BF16, n, rec + 16, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+
+    ft_grad_stats_t stats;
+    ft_step_control_t ctl;
+    HIP_OK(hipMemcpy(&stats, rec, 16, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(&ctl, rec + 16, 16, hipMemcpyDeviceToHost));
+    uint64_t bad = 0;
+    double sumsq = 0;
+    ft_oracle_grad_stats(g.data(), FT_ORACLE_F16, n, 1.f / loss_scale, &bad, &sumsq, 0);
+    check(stats.nonfinite == 0 && bad == 0 && ctl.skip == 0, "statistics: no inf/nan, step not skipped");
+    check(std::fabs(std::sqrt(stats.sumsq) - std::sqrt(sumsq)) <= 1e-6 * std::sqrt(sumsq), "statistics: norm within 1e-6 of the fp64 sum");
+    const float clip = (float)std::fmin(1.0, 1.0 / (std::sqrt(stats.sumsq) + 1e-6));
+    check(ctl.clip_coef == clip && ctl.grad_mult == clip * (1.f / loss_scale) && clip < 1.f, "decision: clip and multiplier follow the closed form");
+
+    ft_oracle_scalars s;
+    ft_oracle_scalars_compute(t, LR, B1, B2, EPS, WD, 1, 1, 0, &s);
+    ft_oracle_adam_step(&s, ctl.grad_mult, p.data(), g.data(), FT_ORACLE_F16, m.data(), v.data(), h.data(), FT_ORACLE_BF16, n, -1, 0);
+    check(same_bits(dp, p) && same_bits(dm, m) && same_bits(dv, v), "update: p, m, v bit-identical to the CPU checker");
+    check(same_bits(dh, h), "update: bf16 copy bit-identical");
+
+    // an overflow: the device-side decision must leave everything untouched
+    const uint16_t inf16 = 0x7c00;
+    HIP_OK(hipMemcpy(dg + 12345, &inf16, 2, hipMemcpyHostToDevice));
+    FT_OK_OR_DIE(ft_grad_stats(dg, FT_F16, n, 1.f / loss_scale, rec, 0, ws, ft_grad_stats_workspace_bytes(), stream));
+    FT_OK_OR_DIE(ft_grad_control(rec, 1.f / loss_scale, 1.0f, rec + 16, stream));
+    FT_OK_OR_DIE(ft_adam_step(7, t + 1, LR, B1, B2, EPS, WD, 1, 1.0f, dp, dg, FT_F16, dm, dv, dh, FT_BF16, n, rec + 16, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(&stats, rec, 16, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(&ctl, rec + 16, 16, hipMemcpyDeviceToHost));
+    check(stats.nonfinite == 1 && ctl.skip == 1, "overflow: one inf counted, skip set");
+    check(same_bits(dp, p) && same_bits(dm, m) && same_bits(dv, v) && same_bits(dh, h), "overflow: state untouched");
+
+    // error behaviour
+    check(ft_adam_step(99, 1, LR, B1, B2, EPS, WD, 1, 1.f, dp, dg, FT_F16, dm, dv, nullptr, FT_BF16, n, nullptr, stream) == FT_ENOENT &&
+              std::strstr(ft_last_error(), "99") != nullptr,
+          "unknown optimizer id is FT_ENOENT with a message");
+    check(ft_adam_step(7, 1, LR, B1, B2, EPS, WD, 1, 1.f, reinterpret_cast<char*>(dp) + 2, dg, FT_F16, dm, dv, nullptr, FT_BF16, 8, nullptr,
+                       stream) == FT_EALIGN,
+          "pointer not aligned to its element is FT_EALIGN");
+    check(ft_adam_step(7, 1, LR, B1, B2, EPS, WD, 1, 1.f, dp, dg, 9, dm, dv, nullptr, FT_BF16, 8, nullptr, stream) == FT_EINVAL,
+          "unknown dtype code is FT_EINVAL");
+    check(ft_adam_step(7, 1, LR, B1, B2, EPS, WD, 1, 1.f, nullptr, nullptr, FT_F32, nullptr, nullptr, nullptr, FT_BF16, 0, nullptr, stream) == FT_OK,
+          "zero elements is a no-op");
+    FT_OK_OR_DIE(ft_adam_destroy(7));
+    // like the reference's erase of a missing key (cpu_adam_impl.cpp:297-302)
+    check(ft_adam_destroy(7) == FT_OK, "destroying an id twice is a harmless no-op");
+    check(ft_adam_step(7, 1, LR, B1, B2, EPS, WD, 1, 1.f, dp, dg, FT_F16, dm, dv, nullptr, FT_BF16, 8, nullptr, stream) == FT_ENOENT,
+          "a destroyed id is unknown afterwards");
+    HIP_OK(hipFree(dp)); HIP_OK(hipFree(dm)); HIP_OK(hipFree(dv)); HIP_OK(hipFree(dg)); HIP_OK(hipFree(dh));
+    HIP_OK(hipFree(ws)); HIP_OK(hipFree(rec));
+}
+
+void accumulate_pass(hipStream_t stream)
+{
+    const size_t n = 300007;
+    Rng rng{7};
+    std::vector<float> acc(n);
+    std::vector<uint16_t> g(n);
+    for (size_t i = 0; i < n; ++i) {
+        acc[i] = rng.normal(1.f);
+        g[i] = ft_oracle_f32_to_bf16(rng.normal(0.1f));
+    }
+    float* dacc = dev_copy(acc);
+    uint16_t* dg = dev_copy(g);
+    void* ws = nullptr;
+    char* rec = nullptr;
+    HIP_OK(hipMalloc(&ws, ft_grad_accumulate_workspace_bytes(n)));
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&rec), 16));
+    FT_OK_OR_DIE(ft_grad_accumulate(dacc, FT_F32, dg, FT_BF16, n, 0.25f, 1, 1.0f, rec, 0, ws, ft_grad_accumulate_workspace_bytes(n), stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    ft_oracle_grad_accumulate(acc.data(), FT_ORACLE_F32, g.data(), FT_ORACLE_BF16, n, 0.25f, 1);
+    check(same_bits(dacc, acc), "accumulate: acc bit-identical to the CPU checker");
+    check(same_bits(dg, g), "accumulate: source cleared");
+    ft_grad_stats_t stats;
+    HIP_OK(hipMemcpy(&stats, rec, 16, hipMemcpyDeviceToHost));
+    uint64_t bad = 0;
+    double sumsq = 0;
+    ft_oracle_grad_stats(acc.data(), FT_ORACLE_F32, n, 1.0f, &bad, &sumsq, 0);
+    check(stats.nonfinite == 0 && std::fabs(stats.sumsq - sumsq) <= 2e-6 * sumsq, "accumulate: fused statistics match");
+    HIP_OK(hipFree(dacc)); HIP_OK(hipFree(dg)); HIP_OK(hipFree(ws)); HIP_OK(hipFree(rec));
+}
+
+void offloaded_step(hipStream_t stream)
+{
+    const size_t n = 3 * (1u << 18) + 1001;  // four chunks, the last one partial
+    Rng rng{99};
+    float *p = nullptr, *m = nullptr, *v = nullptr;
+    FT_OK_OR_DIE(ft_pinned_alloc(n * 4, reinterpret_cast<void**>(&p)));
+    FT_OK_OR_DIE(ft_pinned_alloc(n * 4, reinterpret_cast<void**>(&m)));
+    FT_OK_OR_DIE(ft_pinned_alloc(n * 4, reinterpret_cast<void**>(&v)));
+    std::vector<float> rp(n), rm(n), rv(n);
+    std::vector<uint16_t> g(n), rh(n, 0);
+    for (size_t i = 0; i < n; ++i) {
+        p[i] = rp[i] = rng.normal(0.02f);
+        m[i] = rm[i] = rng.normal(1e-4f);
+        v[i] = rv[i] = (float)(rng.uniform() * 1e-6);
+        g[i] = ft_oracle_f32_to_bf16(rng.normal(1e-3f));
+    }
+    uint16_t *dg = dev_copy(g), *dh = dev_copy(rh);
+    FT_OK_OR_DIE(ft_adam_create(8, LR, B1, B2, EPS, WD, 1, 0));
+    ft_oracle_scalars s;
+    const int modes[] = {FT_OFFLOAD_STAGED, FT_OFFLOAD_DIRECT, FT_OFFLOAD_AUTO};
+    void* eng = nullptr;
+    FT_OK_OR_DIE(ft_offload_create(1u << 18, 3, &eng));
+    for (int k = 0; k < 3; ++k) {
+        const uint64_t t = 10 + k;
+        FT_OK_OR_DIE(ft_offload_set_mode(eng, modes[k]));
+        FT_OK_OR_DIE(ft_offload_step(eng, 8, t, LR, B1, B2, EPS, WD, 1, 1.0f, p, dg, FT_BF16, 0, m, v, dh, FT_BF16, 0, n, nullptr, stream));
+        FT_OK_OR_DIE(ft_offload_wait(eng));
+        ft_oracle_scalars_compute(t, LR, B1, B2, EPS, WD, 1, 1, 0, &s);
+        ft_oracle_adam_step(&s, 1.0f, rp.data(), g.data(), FT_ORACLE_BF16, rm.data(), rv.data(), rh.data(), FT_ORACLE_BF16, n, -1, 0);
+        const bool host_ok = !std::memcmp(p, rp.data(), n * 4) && !std::memcmp(m, rm.data(), n * 4) && !std::memcmp(v, rv.data(), n * 4);
+        char what[96];
+        std::snprintf(what, sizeof what, "offloaded step, mode %d: host p, m, v and device bf16 copy bit-identical", modes[k]);
+        check(host_ok && same_bits(dh, rh), what);
+    }
+    float ms = -1.f;
+    FT_OK_OR_DIE(ft_offload_elapsed_ms(eng, &ms));
+    check(ms > 0.f, "offloaded step reports its device time");
+    FT_OK_OR_DIE(ft_offload_destroy(eng));
+    FT_OK_OR_DIE(ft_adam_destroy(8));
+    FT_OK_OR_DIE(ft_pinned_free(p));
+    FT_OK_OR_DIE(ft_pinned_free(m));
+    FT_OK_OR_DIE(ft_pinned_free(v));
+    HIP_OK(hipFree(dg)); HIP_OK(hipFree(dh));
+}
+
+}  // namespace
+
+int main()
+{
+    std::printf("ft_abi_version %d, devices %d\n", ft_abi_version(), ft_device_count());
+    if (ft_device_count() < 1) {
+        std::printf("FAIL  no GPU visible\n");
+        return 2;
+    }
+    HIP_OK(hipSetDevice(0));
+    hipStream_t stream;
+    HIP_OK(hipStreamCreate(&stream));
+    resident_mixed_precision_step(stream);
+    accumulate_pass(stream);
+    offloaded_step(stream);
+    HIP_OK(hipStreamDestroy(stream));
+    std::printf("%s (%d failed)\n", g_failures ? "FAILED" : "ALL PASSED", g_failures);
+    return g_failures ? 1 : 0;
+}
