@@ -112,6 +112,29 @@ __device__ __forceinline__ void st(T* p, T x)
         *p = x;
 }
 
+// Streaming stores of a whole tile go through buffer instructions, because those let the cache
+// policy be chosen: `nt` (what a non-temporal global store sets) plus agent scope `sc1`, which
+// makes the L2 write the line through instead of holding it dirty. Measured on the update kernel
+// at 2e8 elements: 0.827 ms against 0.842 ms with `nt` alone (`sc0 sc1 nt` the same; no policy on
+// the loads made a difference). The descriptor covers exactly one array's share of the tile
+// (base = wave-uniform tile start, num_records = its bytes), so the hardware also drops any store
+// that would fall outside it.
+constexpr int kAuxStreamStore = 18;  // bit 1: nt, bit 4: sc1
+constexpr int kRawBufferFlags = 0x00027000;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(void* tile_base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(tile_base, 0, (int)bytes, kRawBufferFlags);
+}
+__device__ __forceinline__ void st_stream(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, f32x4 x)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, (int)byte_offset, 0, kAuxStreamStore);
+}
+__device__ __forceinline__ void st_stream(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, u32x2 x)
+{
+    __builtin_amdgcn_raw_buffer_store_b64(x, r, (int)byte_offset, 0, kAuxStreamStore);
+}
+
 // Gradient unit = 4 consecutive elements.
 template <int GT, bool NT>
 __device__ __forceinline__ f32x4 load_g4(const void* g, uint64_t unit)
@@ -177,13 +200,36 @@ __global__ __launch_bounds__(BLOCK) void adam_vec_kernel(AdamArgs a)
             for (int u = 0; u < UNROLL; ++u) {
                 adam_unit(p[u], g[u], m[u], v[u], c);
             }
+            if constexpr (NT_ST) {
+                const uint64_t t0 = tile * kTile;  // first unit of the tile: wave-uniform
+                const __amdgpu_buffer_rsrc_t rp = tile_rsrc(PO + t0, kTile * 16), rm = tile_rsrc(MO + t0, kTile * 16),
+                                             rv = tile_rsrc(VO + t0, kTile * 16);
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint64_t i = base + (uint64_t)u * BLOCK;
-                st<NT_ST>(PO + i, p[u]);
-                st<NT_ST>(MO + i, m[u]);
-                st<NT_ST>(VO + i, v[u]);
-                store_h4<HT, NT_ST>(a.h, i, p[u]);
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint32_t lane_unit = threadIdx.x + (uint32_t)u * BLOCK;
+                    st_stream(rp, lane_unit * 16, p[u]);
+                    st_stream(rm, lane_unit * 16, m[u]);
+                    st_stream(rv, lane_unit * 16, v[u]);
+                }
+                if constexpr (HT == FT_F16 || HT == FT_BF16) {
+                    const __amdgpu_buffer_rsrc_t rh = tile_rsrc(reinterpret_cast<u32x2*>(a.h) + t0, kTile * 8);
+#pragma unroll
+                    for (int u = 0; u < UNROLL; ++u) {
+                        u32x2 w;
+                        w.x = pack2<HT>(p[u].x, p[u].y);
+                        w.y = pack2<HT>(p[u].z, p[u].w);
+                        st_stream(rh, (threadIdx.x + (uint32_t)u * BLOCK) * 8, w);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) {
+                    const uint64_t i = base + (uint64_t)u * BLOCK;
+                    PO[i] = p[u];
+                    MO[i] = m[u];
+                    VO[i] = v[u];
+                    store_h4<HT, false>(a.h, i, p[u]);
+                }
             }
         } else {  // last, partial tile
             for (int u = 0; u < UNROLL; ++u) {
@@ -439,13 +485,22 @@ __device__ __forceinline__ void stats_of_stored(float value, uint32_t bits, floa
     acc = __builtin_fmaf(nf ? 0.0f : x, nf ? 0.0f : x, acc);
 }
 
+// One 64-unit tile: lane `threadIdx.x` takes unit tile*64 + lane when that is below nvec. All
+// accesses are streaming: every buffer is far larger than the caches and is touched once. The
+// descriptors cover only the units of this tile that exist, so lanes past nvec cannot store.
 template <int AT, int GT, bool ZERO, bool STATS>
-__device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, float scale, float pre_mult,
-                                                float (&sums)[4], uint32_t& bad)
+__device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t tile, uint64_t nvec, float scale,
+                                                float pre_mult, float (&sums)[4], uint32_t& bad)
 {
+    constexpr uint32_t kAccUnit = (AT == FT_F32) ? 16 : 8, kGradUnit = (GT == FT_F32) ? 16 : 8;
+    const uint64_t t0 = tile * 64;  // wave-uniform
+    const uint32_t live = (nvec - t0 < 64) ? (uint32_t)(nvec - t0) : 64u;
+    const __amdgpu_buffer_rsrc_t racc = tile_rsrc(static_cast<char*>(acc) + t0 * kAccUnit, live * kAccUnit);
+    const uint64_t i = t0 + threadIdx.x;
+    if (threadIdx.x >= live) return;
+
     const f32x4 g4 = load_g4<GT, true>(g, i);
     f32x4 a4;
-    // Streaming accesses throughout: every buffer is far larger than the caches and is touched once.
     if constexpr (AT == FT_F32) {
         a4 = ld<true>(reinterpret_cast<const f32x4*>(acc) + i);
     } else {
@@ -463,7 +518,7 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
         r[k] = x;
     }
     if constexpr (AT == FT_F32) {
-        st<true>(reinterpret_cast<f32x4*>(acc) + i, r);
+        st_stream(racc, threadIdx.x * kAccUnit, r);
         if constexpr (STATS) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -475,7 +530,7 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
         u32x2 w;
         w.x = pack2<AT>(r.x, r.y);
         w.y = pack2<AT>(r.z, r.w);
-        st<true>(reinterpret_cast<u32x2*>(acc) + i, w);
+        st_stream(racc, threadIdx.x * kAccUnit, w);
         if constexpr (STATS) {
             const uint32_t b[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
 #pragma unroll
@@ -483,12 +538,13 @@ __device__ __forceinline__ void accumulate_unit(void* acc, void* g, uint64_t i, 
         }
     }
     if constexpr (ZERO) {
+        const __amdgpu_buffer_rsrc_t rg = tile_rsrc(static_cast<char*>(g) + t0 * kGradUnit, live * kGradUnit);
         if constexpr (GT == FT_F32) {
             const f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            st<true>(reinterpret_cast<f32x4*>(g) + i, z);
+            st_stream(rg, threadIdx.x * kGradUnit, z);
         } else {
             const u32x2 z = {0u, 0u};
-            st<true>(reinterpret_cast<u32x2*>(g) + i, z);
+            st_stream(rg, threadIdx.x * kGradUnit, z);
         }
     }
 }
@@ -507,9 +563,9 @@ __global__ __launch_bounds__(64) void grad_accumulate_kernel(void* acc, void* g,
 {
     float sums[4] = {0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
-    const uint64_t stride = (uint64_t)gridDim.x * 64;
-    for (uint64_t i = (uint64_t)blockIdx.x * 64 + threadIdx.x; i < nvec; i += stride)
-        accumulate_unit<AT, GT, ZERO, STATS>(acc, g, i, scale, pre_mult, sums, bad);
+    const uint64_t ntiles = (nvec + 63) / 64;
+    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x)
+        accumulate_tile<AT, GT, ZERO, STATS>(acc, g, tile, nvec, scale, pre_mult, sums, bad);
     if constexpr (STATS) {
         const float t = wave_sum((sums[0] + sums[1]) + (sums[2] + sums[3]));
         const uint32_t tb = wave_sum_u32(bad);
