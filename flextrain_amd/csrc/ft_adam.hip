@@ -322,7 +322,7 @@ size_t accumulate_workspace_bytes(size_t n)
 
 template <int AT, int GT, bool ZERO, bool STATS>
 int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, float scale, float pre_mult,
-                      ftk::StatsPartial* parts, int* nparts, hipStream_t stream)
+                      ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, hipStream_t stream)
 {
     constexpr size_t asz = (AT == FT_F32) ? 4 : 2, gsz = (GT == FT_F32) ? 4 : 2;
     int reduce_blocks = 0;
@@ -348,35 +348,36 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
             FT_HIP(hipGetLastError());
         }
     }
+    // Edge elements and, with statistics, the sum of the second-level partials: one small launch.
     const size_t tail_begin = head + nvec * 4;
     if (STATS || head > 0 || tail_begin < n) {
-        hipLaunchKernelGGL((ftk::grad_accumulate_edge_kernel<AT, GT, ZERO, STATS>), dim3(1), dim3(64), 0, stream, acc, g,
+        hipLaunchKernelGGL((ftk::grad_accumulate_finish_kernel<AT, GT, ZERO, STATS>), dim3(1), dim3(256), 0, stream, acc, g,
                            static_cast<uint64_t>(head), static_cast<uint64_t>(tail_begin), static_cast<uint64_t>(n),
-                           scale, pre_mult, parts + reduce_blocks);
+                           scale, pre_mult, static_cast<const ftk::StatsPartial*>(parts), reduce_blocks, stats_out,
+                           stats_accumulate);
         FT_HIP(hipGetLastError());
     }
-    *nparts = reduce_blocks + 1;
     return FT_OK;
 }
 
 template <int AT, int GT>
 int launch_accumulate_flags(bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec, float scale,
-                            float pre_mult, ftk::StatsPartial* parts, int* nparts, hipStream_t stream)
+                            float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, hipStream_t stream)
 {
-    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
-    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
-    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
-    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
+    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
+    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
+    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
+    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
 }
 
 template <int AT>
 int launch_accumulate_g(int g_dtype, bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec,
-                        float scale, float pre_mult, ftk::StatsPartial* parts, int* nparts, hipStream_t stream)
+                        float scale, float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, hipStream_t stream)
 {
     switch (g_dtype) {
-        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
-        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
-        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, nparts, stream);
+        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
+        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
+        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
     }
 }
 
@@ -533,22 +534,12 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
         int wrc = resolve_stats_workspace(workspace, workspace_bytes, accumulate_workspace_bytes(n), &parts);
         if (wrc != FT_OK) return wrc;
     }
-    int nparts = 0;
-    int rc;
+    ft_grad_stats_t* out = static_cast<ft_grad_stats_t*>(stats_out);
     switch (acc_dtype) {
-        case FT_F32: rc = launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, &nparts, stream); break;
-        case FT_F16: rc = launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, &nparts, stream); break;
-        default: rc = launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, &nparts, stream); break;
+        case FT_F32: return launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
+        case FT_F16: return launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
+        default: return launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
     }
-    if (rc != FT_OK) return rc;
-    if (stats) {
-        // second-level partials plus the edge kernel's one
-        hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, nparts,
-                           static_cast<const void*>(nullptr), static_cast<uint64_t>(0), static_cast<uint64_t>(0),
-                           static_cast<uint64_t>(0), 1.0f, static_cast<ft_grad_stats_t*>(stats_out), stats_accumulate);
-        FT_HIP(hipGetLastError());
-    }
-    return FT_OK;
 }
 
 int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ctl_out, void* stream)

@@ -613,15 +613,19 @@ __global__ __launch_bounds__(256) void reduce_wave_partials_kernel(const WavePar
     }
 }
 
-// Elements outside the vector body, one by one, by a single thread; writes one more partial.
+// Last launch of an accumulation pass (one block of 256): thread 0 takes the elements outside the
+// vector body one by one; with STATS the block then adds the second-level partials in a fixed tree
+// order, thread 0 adds the edge elements' share and writes or accumulates the result.
 template <int AT, int GT, bool ZERO, bool STATS>
-__global__ void grad_accumulate_edge_kernel(void* acc, void* g, uint64_t head, uint64_t tail_begin, uint64_t n,
-                                            float scale, float pre_mult, StatsPartial* partial)
+__global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, void* g, uint64_t head,
+                                                                     uint64_t tail_begin, uint64_t n, float scale,
+                                                                     float pre_mult,
+                                                                     const StatsPartial* __restrict__ partials,
+                                                                     int nparts, ft_grad_stats_t* out, int accumulate)
 {
-    if (threadIdx.x != 0 || blockIdx.x != 0) return;
     double s = 0.0;
     uint64_t b = 0;
-    for (uint64_t i = 0; i < n; ++i) {
+    for (uint64_t i = 0; threadIdx.x == 0 && i < n; ++i) {
         if (i == head) i = tail_begin;
         if (i >= n) break;
         float gi;
@@ -662,8 +666,35 @@ __global__ void grad_accumulate_edge_kernel(void* acc, void* g, uint64_t head, u
         }
     }
     if constexpr (STATS) {
-        partial->sumsq = s;
-        partial->nonfinite = b;
+        __shared__ double s_sum[256];
+        __shared__ uint64_t s_bad[256];
+        double ps = 0.0;
+        uint64_t pb = 0;
+        for (int i = threadIdx.x; i < nparts; i += 256) {
+            ps += partials[i].sumsq;
+            pb += partials[i].nonfinite;
+        }
+        s_sum[threadIdx.x] = ps;
+        s_bad[threadIdx.x] = pb;
+        __syncthreads();
+        for (int w = 128; w > 0; w >>= 1) {
+            if ((int)threadIdx.x < w) {
+                s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
+                s_bad[threadIdx.x] += s_bad[threadIdx.x + w];
+            }
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) {
+            s += s_sum[0];
+            b += s_bad[0];
+            if (accumulate) {
+                out->sumsq += s;
+                out->nonfinite += b;
+            } else {
+                out->sumsq = s;
+                out->nonfinite = b;
+            }
+        }
     }
 }
 
