@@ -209,6 +209,37 @@ def test_steps_on_disjoint_memory_overlap_and_same_memory_stay_ordered(cuda, ora
         _assert_equal_bits(f"unit {u}", p, m, v, halves[u], want[u], torch.bfloat16)
 
 
+@pytest.mark.parametrize("mode", [1, 2])
+def test_buffers_poisoned_as_soon_as_the_engine_says_they_are_free(cuda, oracle, mode):
+    """Event dependencies of the streamed step, made visible with poison. The gradient buffer is
+    filled by a copy enqueued just before the step (the step must wait for its producer), is
+    overwritten with NaN right after a device-side wait for the step's kernels (nothing may read it
+    after that), and the host arrays are read back by a copy ordered only by the device-side wait
+    for the write-back. 46 chunks through 2 slots, no host synchronisation until the end."""
+    from flextrain_amd import FlexTrainCPUAdam
+    n = 3_000_001
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 16, offload_slots=2, offload_mode=mode, **HP)
+    p, m, v = _host_state(n, seed=77)
+    real = (torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16)
+    want = _oracle(oracle, p, real, m, v, 2, torch.bfloat16)
+    g = torch.full((n,), float("nan"), dtype=torch.bfloat16, device=cuda)
+    h = torch.full((n,), float("nan"), dtype=torch.bfloat16, device=cuda)
+    mirror = torch.zeros(n, device=cuda)
+    torch.cuda.synchronize()
+    g.copy_(real)                                   # producer on the current stream
+    eng._step({"step": 2}, h, p, g, m, v, blocking=False)
+    eng.stream_wait()                               # kernels done -> g is free, h is final
+    g.fill_(float("nan"))                           # poison
+    h_seen = h.clone()
+    eng.stream_wait(write_back=True)                # write-back done -> host arrays are final
+    mirror.copy_(p, non_blocking=True)
+    torch.cuda.synchronize()
+    eng.synchronize()
+    _assert_equal_bits(f"poison mode={mode}", p, m, v, h_seen, want, torch.bfloat16)
+    assert torch.equal(mirror.cpu(), p)
+    assert torch.isnan(g).all()
+
+
 def test_config5_offloaded_7b_optimizer(cuda, oracle):
     """The offloaded Llama-7B optimizer at the largest size this machine can pin (all 32 layers +
     embedding + lm_head = 6.74e9 elements need 81 GB of pinned memory; a machine that refuses that
