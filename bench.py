@@ -320,7 +320,8 @@ def bench_pipeline(args, torch, dev) -> int:
         opt.cpu_optimizer._offload_slots = args.slots
         try:
             coord = FlexTrainOptsCoordinator()
-            coord.initialize(opt, flat, mb, offload=True)
+            coord.initialize(opt, flat, mb, offload=True, unit_windows=args.windows != "off",
+                             window_write_through=args.windows == "write_through")
         except _C.FtError:
             coord = None
             del opt, flat, params
@@ -366,7 +367,7 @@ def bench_pipeline(args, torch, dev) -> int:
         "config": {"workload": f"pipeline: coordinator schedule over {units} Llama-7B layers, {mb} shares per unit, "
                                "fp32 state in pinned host DRAM, bf16 grads and parameters on GPU",
                    "elements": total, "units": units, "micro_batches": mb, "chunk_elems": args.chunk_elems,
-                   "slots": args.slots},
+                   "slots": args.slots, "unit_windows": args.windows},
         "link": {"measured_h2d_gbps": link["h2d"], "measured_d2h_gbps": link["d2h"],
                  "measured_bidirectional_gbps": link["both"], "achieved_each_way_gbps": one_way,
                  "achieved_total_gbps": 2 * one_way, "frac_of_unidirectional": one_way / min(link["h2d"], link["d2h"]),
@@ -385,6 +386,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate"])
     ap.add_argument("--micro-batches", type=int, default=4, help="pipeline: shares per unit")
+    ap.add_argument("--windows", default="off", choices=["off", "write_through", "copy_back"],
+                    help="pipeline: keep a whole unit's state on the GPU while it is stepped (prefetched one unit ahead)")
     ap.add_argument("--chunk-elems", type=int, default=64 * 1024 * 1024, help="cfg5: elements per streamed chunk")
     ap.add_argument("--slots", type=int, default=3, help="cfg5: device buffer sets of the pipeline")
     ap.add_argument("--layers", type=int, default=32, help="cfg5: decoder layers (32 = the full 7B optimizer)")

@@ -41,6 +41,8 @@ EXPORTS = {
     "ft_offload_step": (c_int, [c_void_p, c_int, c_uint64, c_float, c_float, c_float, c_float, c_float, c_int,
                                 c_float, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                 c_int, c_size_t, c_void_p, c_void_p]),
+    "ft_offload_window_open": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_int, POINTER(c_int)]),
+    "ft_offload_window_close": (c_int, [c_void_p, c_int]),
     "ft_offload_stream_wait": (c_int, [c_void_p, c_void_p, c_int]),
     "ft_offload_wait": (c_int, [c_void_p]),
     "ft_offload_elapsed_ms": (c_int, [c_void_p, POINTER(c_float)]),

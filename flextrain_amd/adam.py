@@ -196,6 +196,31 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             # later work on the caller's stream may overwrite the gradients or read the new copy
             _C.check("ft_offload_stream_wait", self._lib.ft_offload_stream_wait(engine, _C.current_stream_ptr(), 0))
 
+    def open_window(self, full_parameter: Tensor, exp_avg: Tensor, exp_avg_sq: Tensor, write_through: bool = False) -> int:
+        """Brings the whole master state of one unit (three pinned host tensors of equal length) to
+        the GPU with large copies and keeps it there until ``close_window``: every ``_step`` on
+        slices of these tensors in between is a plain in-place kernel on the device copy, and the
+        host tensors are stale until the close has written them back (``synchronize()`` or
+        ``stream_wait(write_back=True)`` after the close). For callers that step a unit in many
+        small shares, where one copy per share would use the link badly. Returns a token."""
+        n = full_parameter.numel()
+        for name, t in (("full_parameter", full_parameter), ("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq)):
+            _flat(name, t, {torch.float32}, n)
+            if t.is_cuda or not t.is_pinned():
+                raise ValueError(f"{name} must be pinned host memory")
+        token = ctypes.c_int(-1)
+        _C.check("ft_offload_window_open", self._lib.ft_offload_window_open(
+            self._offload_engine(), full_parameter.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n,
+            int(bool(write_through)), ctypes.byref(token)))
+        # the engine holds raw addresses: keep the tensors alive until the write-back is enqueued
+        self.__dict__.setdefault("_window_tensors", {})[int(token.value)] = (full_parameter, exp_avg, exp_avg_sq)
+        return int(token.value)
+
+    def close_window(self, token: int) -> None:
+        """Enqueues the write-back of a window opened with ``open_window`` and returns."""
+        _C.check("ft_offload_window_close", self._lib.ft_offload_window_close(self._offload_engine(), int(token)))
+        self.__dict__.get("_window_tensors", {}).pop(int(token), None)
+
     def synchronize(self):
         """Waits for every offloaded step enqueued so far (no-op if none was)."""
         if self._engine is not None:

@@ -43,6 +43,35 @@ struct Pending {
 
 constexpr size_t kMaxPending = 8;
 
+// A window keeps the whole state of one unit on the device between ft_offload_window_open and
+// ft_offload_window_close: one large H2D per array when it opens (in pieces, each with its own
+// event, so that a step on the front of the unit need not wait for the back), any number of steps
+// on sub-ranges that run as plain kernels on the device copy, and the way back either as one large
+// D2H per array when it closes or -- write_through -- by the step kernels themselves, which then
+// write their results straight to the host arrays (each element may then be stepped once per
+// window). Measured on the 24-layer schedule with 16 shares per unit (each way, concurrently):
+// per-share direct 43.5 GB/s; write-through windows 44.5 GB/s, every iteration alike; copy-back
+// windows 47.7 GB/s in most iterations but 28 GB/s in about one of six, when copies that were
+// enqueued long before their dependencies resolved end up queued behind one another on one copy
+// engine (waiting on the host until a copy can start removes those iterations, at the price of a
+// host-device synchronisation per unit, which a training loop cannot afford).
+constexpr size_t kWindowPieceElems = 64u * 1024u * 1024u;  // about 256 MiB per array and copy
+constexpr int kMaxWindows = 4;
+
+struct Window {
+    float* dev[3] = {nullptr, nullptr, nullptr};
+    size_t cap = 0;                  // elements each device array can hold
+    uintptr_t host[3] = {0, 0, 0};   // host arrays this window mirrors while open
+    size_t n = 0;
+    bool open = false;
+    bool used = false;               // d2h_done has been recorded at least once
+    bool write_through = false;      // steps write their results to the host arrays themselves
+    size_t piece = 0;                // elements per copy: n cut into equal pieces, never a small tail
+    uint64_t closed_at = 0;          // order of closing: the window closed longest ago is reused first
+    std::vector<hipEvent_t> piece_done;
+    hipEvent_t k_done = nullptr, d2h_done = nullptr;
+};
+
 // Automatic choice of the transfer mode. Measured on MI355X / PCIe Gen5 x16: SDMA copies through
 // staging slots move 48-49 GB/s each way when every copy is at least ~128 MiB, but a run of many
 // smaller copies ends up with both directions on one SDMA engine and drops to 15 GB/s; the kernel
@@ -64,6 +93,8 @@ struct Engine {
     int mode = FT_OFFLOAD_AUTO;
     std::deque<Pending> recent;        // steps whose write-back may still be in flight, oldest first
     std::vector<hipEvent_t> free_events;
+    Window windows[kMaxWindows];
+    uint64_t window_closes = 0;
 };
 
 Engine* as_engine(void* h)
@@ -108,8 +139,70 @@ void destroy_engine(Engine* e)
     for (Pending& pd : e->recent)
         if (pd.done) (void)hipEventDestroy(pd.done);
     for (hipEvent_t ev : e->free_events) (void)hipEventDestroy(ev);
+    for (Window& w : e->windows) {
+        for (float* d : w.dev)
+            if (d) (void)hipFree(d);
+        for (hipEvent_t ev : w.piece_done) (void)hipEventDestroy(ev);
+        if (w.k_done) (void)hipEventDestroy(w.k_done);
+        if (w.d2h_done) (void)hipEventDestroy(w.d2h_done);
+    }
     e->magic = 0;
     delete e;
+}
+
+// Orders the H2D and kernel streams behind the newest earlier write-back that touched any of the
+// host ranges in `mine` (the D2H stream is in order, so that one event covers all older ones).
+int wait_for_overlapping_writebacks(Engine* e, const Pending& mine)
+{
+    for (auto it = e->recent.rbegin(); it != e->recent.rend(); ++it) {
+        if (it->overlaps(mine)) {
+            FT_HIP(hipStreamWaitEvent(e->s_h2d, it->done, 0));
+            FT_HIP(hipStreamWaitEvent(e->s_k, it->done, 0));
+            break;
+        }
+    }
+    return FT_OK;
+}
+
+// Remembers a write-back whose last D2H is the newest work on the D2H stream. When the list is
+// full the oldest entry is retired; every later H2D is then ordered behind it, which costs
+// nothing once it has long finished.
+int remember_writeback(Engine* e, Pending mine)
+{
+    if (e->free_events.empty()) {
+        Pending& old = e->recent.front();
+        FT_HIP(hipStreamWaitEvent(e->s_h2d, old.done, 0));
+        FT_HIP(hipStreamWaitEvent(e->s_k, old.done, 0));
+        e->free_events.push_back(old.done);
+        e->recent.pop_front();
+    }
+    mine.done = e->free_events.back();
+    e->free_events.pop_back();
+    FT_HIP(hipEventRecord(mine.done, e->s_d2h));
+    e->recent.push_back(mine);
+    return FT_OK;
+}
+
+// The open window that holds [host_p, host_p + n) and the matching ranges of m and v, if any.
+// Returns FT_OK with *out = nullptr when no window is involved, an error for a partial overlap.
+int find_window(Engine* e, const void* host_p, const void* host_m, const void* host_v, size_t n, Window** out, size_t* off)
+{
+    *out = nullptr;
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(host_p), hi = lo + n * 4;
+    for (Window& w : e->windows) {
+        if (!w.open) continue;
+        const uintptr_t wlo = w.host[0], whi = w.host[0] + w.n * 4;
+        if (hi <= wlo || whi <= lo) continue;
+        if (lo < wlo || hi > whi)
+            return fth::fail(FT_EINVAL, "a step must lie entirely inside or entirely outside an open window");
+        const size_t o = (lo - wlo) / 4;
+        if (reinterpret_cast<uintptr_t>(host_m) != w.host[1] + o * 4 || reinterpret_cast<uintptr_t>(host_v) != w.host[2] + o * 4)
+            return fth::fail(FT_EINVAL, "exp_avg / exp_avg_sq are not at the params' offset inside the open window");
+        *out = &w;
+        *off = o;
+        return FT_OK;
+    }
+    return FT_OK;
 }
 
 }  // namespace
@@ -214,6 +307,10 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     if (g_on_host && (rc = require_pinned(g, "grads")) != FT_OK) return rc;
     if (half_out && half_on_host && (rc = require_pinned(half_out, "low-precision copy")) != FT_OK) return rc;
 
+    Window* window = nullptr;
+    size_t window_off = 0;
+    if ((rc = find_window(e, host_p, host_m, host_v, n, &window, &window_off)) != FT_OK) return rc;
+
     const size_t gsz = g_dtype == FT_F32 ? 4 : 2;
     const size_t chunk = e->chunk;
     const ftk::AdamConsts c =
@@ -235,17 +332,36 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     if (half_out && half_on_host) add_range(half_out, n * 2);
 
     // The pipeline starts after the producer of g/ctl on the caller's stream ...
+    // (a step inside a window copies nothing, so the H2D stream, which may be prefetching the next
+    // window, is left alone)
     FT_HIP(hipEventRecord(e->ev_user, user));
-    FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_user, 0));
+    if (!window) FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_user, 0));
     FT_HIP(hipStreamWaitEvent(e->s_k, e->ev_user, 0));
     // ... and after the newest earlier step that wrote to the same host memory (the D2H stream is
     // in order, so that one event covers all older ones).
-    for (auto it = e->recent.rbegin(); it != e->recent.rend(); ++it) {
-        if (it->overlaps(mine)) {
-            FT_HIP(hipStreamWaitEvent(e->s_h2d, it->done, 0));
-            FT_HIP(hipStreamWaitEvent(e->s_k, it->done, 0));
-            break;
+    if (!window && (rc = wait_for_overlapping_writebacks(e, mine)) != FT_OK) return rc;
+
+    // State held in an open window: the step is one in-place kernel on the device copy; nothing
+    // crosses the link until the window closes.
+    if (window) {
+        const size_t last_piece = (window_off + n - 1) / window->piece;
+        FT_HIP(hipStreamWaitEvent(e->s_k, window->piece_done[last_piece], 0));
+        FT_HIP(hipEventRecord(e->ev_begin, e->s_k));
+        float* out[3] = {nullptr, nullptr, nullptr};  // nullptr = in place on the device copy
+        if (window->write_through) {
+            out[0] = static_cast<float*>(host_p);
+            out[1] = static_cast<float*>(host_m);
+            out[2] = static_cast<float*>(host_v);
         }
+        rc = fth::launch_adam(c, window->dev[0] + window_off, g, g_dtype, window->dev[1] + window_off,
+                              window->dev[2] + window_off, half_out, half_dtype, n,
+                              static_cast<const ft_step_control_t*>(ctl), e->s_k, out[0], out[1], out[2]);
+        if (rc != FT_OK) return rc;
+        FT_HIP(hipEventRecord(e->ev_kernels, e->s_k));
+        FT_HIP(hipStreamWaitEvent(e->s_d2h, e->ev_kernels, 0));
+        FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
+        e->stepped = true;
+        return FT_OK;
     }
     FT_HIP(hipEventRecord(e->ev_begin, e->s_h2d));
 
@@ -325,20 +441,126 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
     e->stepped = true;
 
-    // Remember this step's write-back. When the list is full the oldest entry is retired; every
-    // later H2D is then ordered behind it, which costs nothing once it has long finished.
-    if (e->free_events.empty()) {
-        Pending& old = e->recent.front();
-        FT_HIP(hipStreamWaitEvent(e->s_h2d, old.done, 0));
-        FT_HIP(hipStreamWaitEvent(e->s_k, old.done, 0));
-        e->free_events.push_back(old.done);
-        e->recent.pop_front();
+    return remember_writeback(e, mine);
+}
+
+int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_v, size_t n, int write_through,
+                           int* out_window)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    if (!out_window) return fth::fail(FT_EINVAL, "out_window must not be NULL");
+    *out_window = -1;
+    if (n == 0 || !host_p || !host_m || !host_v) return fth::fail(FT_EINVAL, "p, m, v must not be NULL and n must be positive");
+    int rc;
+    if ((rc = require_pinned(host_p, "params")) != FT_OK) return rc;
+    if ((rc = require_pinned(host_m, "exp_avg")) != FT_OK) return rc;
+    if ((rc = require_pinned(host_v, "exp_avg_sq")) != FT_OK) return rc;
+    void* host[3] = {host_p, host_m, host_v};
+    Pending mine;
+    for (int a = 0; a < 3; ++a) {
+        mine.lo[a] = reinterpret_cast<uintptr_t>(host[a]);
+        mine.hi[a] = mine.lo[a] + n * 4;
     }
-    mine.done = e->free_events.back();
-    e->free_events.pop_back();
-    FT_HIP(hipEventRecord(mine.done, e->s_d2h));
-    e->recent.push_back(mine);
+    mine.ranges = 3;
+    for (Window& w : e->windows) {
+        if (!w.open) continue;
+        for (int a = 0; a < 3; ++a)
+            for (int b = 0; b < 3; ++b)
+                if (mine.lo[a] < w.host[b] + w.n * 4 && w.host[b] < mine.hi[a])
+                    return fth::fail(FT_EBUSY, "this host memory already belongs to an open window");
+    }
+    // The window that was closed longest ago (its write-back has had the most time to finish, and
+    // the new copies must wait for it); never-used ones first.
+    int pick = -1;
+    for (int i = 0; i < kMaxWindows; ++i) {
+        const Window& w = e->windows[i];
+        if (w.open) continue;
+        if (pick < 0 || w.closed_at < e->windows[pick].closed_at) pick = i;
+    }
+    if (pick < 0) return fth::fail(FT_EBUSY, "all %d windows are open", kMaxWindows);
+    Window& w = e->windows[pick];
+    if (!w.k_done) FT_HIP(hipEventCreateWithFlags(&w.k_done, hipEventDisableTiming));
+    if (!w.d2h_done) FT_HIP(hipEventCreateWithFlags(&w.d2h_done, hipEventDisableTiming));
+    if (w.cap < n) {
+        if (w.used) FT_HIP(hipEventSynchronize(w.d2h_done));  // its last write-back still reads the old arrays
+        for (float*& d : w.dev) {
+            if (d) FT_HIP(hipFree(d));
+            d = nullptr;
+        }
+        w.cap = 0;
+        for (float*& d : w.dev) {
+            hipError_t err = hipMalloc(reinterpret_cast<void**>(&d), n * 4);
+            if (err != hipSuccess) {
+                (void)hipGetLastError();
+                return fth::fail(FT_ENOMEM, "hipMalloc(%zu) for a window failed: %s", n * 4, hipGetErrorString(err));
+            }
+        }
+        w.cap = n;
+    }
+    // Equal pieces of about kWindowPieceElems: a short last copy would be one of the small copies
+    // that make the copy engines share (see kStagedMinElems).
+    size_t pieces = (n + kWindowPieceElems / 2) / kWindowPieceElems;
+    if (pieces == 0) pieces = 1;
+    const size_t piece = ((n + pieces - 1) / pieces + 3) / 4 * 4;
+    pieces = (n + piece - 1) / piece;
+    while (w.piece_done.size() < pieces) {
+        hipEvent_t ev = nullptr;
+        FT_HIP(hipEventCreateWithFlags(&ev, hipEventDisableTiming));
+        w.piece_done.push_back(ev);
+    }
+    // The copies read host memory: behind any write-back to it that is still in flight, and behind
+    // the window's own previous write-back, which still reads the device arrays.
+    if ((rc = wait_for_overlapping_writebacks(e, mine)) != FT_OK) return rc;
+    if (w.used) FT_HIP(hipStreamWaitEvent(e->s_h2d, w.d2h_done, 0));
+    for (size_t k = 0; k < pieces; ++k) {
+        const size_t off = k * piece;
+        const size_t cnt = (n - off < piece) ? (n - off) : piece;
+        for (int a = 0; a < 3; ++a)
+            FT_HIP(hipMemcpyAsync(w.dev[a] + off, static_cast<float*>(host[a]) + off, cnt * 4, hipMemcpyHostToDevice, e->s_h2d));
+        FT_HIP(hipEventRecord(w.piece_done[k], e->s_h2d));
+    }
+    for (int a = 0; a < 3; ++a) w.host[a] = reinterpret_cast<uintptr_t>(host[a]);
+    w.n = n;
+    w.piece = piece;
+    w.write_through = write_through != 0;
+    w.open = true;
+    *out_window = pick;
     return FT_OK;
+}
+
+int ft_offload_window_close(void* handle, int window)
+{
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    if (window < 0 || window >= kMaxWindows || !e->windows[window].open)
+        return fth::fail(FT_ENOENT, "window %d is not open", window);
+    Window& w = e->windows[window];
+    // Everything the kernel stream holds so far includes every step on this window.
+    FT_HIP(hipEventRecord(w.k_done, e->s_k));
+    FT_HIP(hipStreamWaitEvent(e->s_d2h, w.k_done, 0));
+    // A window nobody stepped in still has its copies in flight; they must land before the way back.
+    const size_t pieces = (w.n + w.piece - 1) / w.piece;
+    FT_HIP(hipStreamWaitEvent(e->s_d2h, w.piece_done[pieces - 1], 0));
+    Pending mine;
+    for (size_t k = 0; k < pieces && !w.write_through; ++k) {
+        const size_t off = k * w.piece;
+        const size_t cnt = (w.n - off < w.piece) ? (w.n - off) : w.piece;
+        for (int a = 0; a < 3; ++a)
+            FT_HIP(hipMemcpyAsync(reinterpret_cast<float*>(w.host[a]) + off, w.dev[a] + off, cnt * 4, hipMemcpyDeviceToHost, e->s_d2h));
+    }
+    FT_HIP(hipEventRecord(w.d2h_done, e->s_d2h));
+    FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
+    e->stepped = true;
+    for (int a = 0; a < 3; ++a) {
+        mine.lo[a] = w.host[a];
+        mine.hi[a] = w.host[a] + w.n * 4;
+    }
+    mine.ranges = 3;
+    w.open = false;
+    w.used = true;
+    w.closed_at = ++e->window_closes;
+    return remember_writeback(e, mine);
 }
 
 int ft_offload_set_mode(void* handle, int mode)

@@ -172,6 +172,20 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
                     void* host_p, const void* g, int g_dtype, int g_on_host, void* host_m,
                     void* host_v, void* half_out, int half_dtype, int half_on_host, size_t n,
                     const void* ctl, void* stream);
+/* Windows: where a caller steps one unit's state in many small pieces (the per-(unit, micro-batch)
+ * calls of flextrain/memory/coordinator/optimizer.py:684-696), copies of a few tens of MB each use
+ * the link badly. ft_offload_window_open brings the whole p, m, v of the unit (n elements each) to
+ * the device with large copies and returns at once; until ft_offload_window_close, every
+ * ft_offload_step whose p/m/v lie inside those arrays (same element offset in all three) runs as
+ * a kernel on the device copy. write_through == 0: the kernels work in place on the device copy,
+ * the host arrays are stale until the close has written all three back with large copies.
+ * write_through != 0: the kernels write their results straight to the host arrays (no copy back;
+ * each element may be stepped at most once per window). A step may not straddle a window's edge.
+ * At most 4 windows are open at a time (FT_EBUSY beyond). The reference has no counterpart: its
+ * state never leaves the host. */
+int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_v, size_t n, int write_through,
+                           int* out_window);
+int ft_offload_window_close(void* handle, int window);
 int ft_offload_stream_wait(void* handle, void* stream, int what);
 int ft_offload_wait(void* handle);
 int ft_offload_elapsed_ms(void* handle, float* out_ms);

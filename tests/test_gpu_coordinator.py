@@ -15,8 +15,8 @@ class _Unit:
         self.paras = paras
 
 
-@pytest.mark.parametrize("offload", [True, False])
-def test_backward_pipeline_matches_oracle(cuda, oracle, offload):
+@pytest.mark.parametrize("offload,windows", [(True, "copy_back"), (True, "write_through"), (True, None), (False, None)])
+def test_backward_pipeline_matches_oracle(cuda, oracle, offload, windows):
     from flextrain_amd import FlexTrainAdam
     from flextrain_amd.coordinator import FlexTrainOptsCoordinator
     torch.manual_seed(0)
@@ -38,7 +38,8 @@ def test_backward_pipeline_matches_oracle(cuda, oracle, offload):
     assert opt.non_layerwise_numel == 0
     assert [(s.start, s.end) for s in opt.unit_group_segments[0]] == [(0, w_numel), (w_numel, unit_numel)]
     coord = FlexTrainOptsCoordinator()
-    coord.initialize(opt, flat, micro_batches, offload=offload)
+    coord.initialize(opt, flat, micro_batches, offload=offload, unit_windows=windows is not None,
+                     window_write_through=windows == "write_through")
     assert coord.unit_master_parameter(0).is_pinned() == offload
 
     # oracle state, seeded the same way
@@ -71,7 +72,7 @@ def test_backward_pipeline_matches_oracle(cuda, oracle, offload):
             m, v = coord.unit_optimizer_states(u)
             worst = dict(p=max_ulp(to_np(coord.unit_master_parameter(u)), pn), m=max_ulp(to_np(m), mn),
                          v=max_ulp(to_np(v), vn), h=max_ulp(half_bits(flat[u]), hn, bf16=True))
-            print(f"[coordinator offload={offload} it={iteration} unit={u}] worst ULP distance: {worst}", flush=True)
+            print(f"[coordinator offload={offload} windows={windows} it={iteration} unit={u}] worst ULP distance: {worst}", flush=True)
             assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst["h"] <= HALF_ULP
     assert decay["step"] == 2 and plain["step"] == 2
     # the module's parameters are views of the flat unit buffers: they saw the update

@@ -240,6 +240,90 @@ def test_buffers_poisoned_as_soon_as_the_engine_says_they_are_free(cuda, oracle,
     assert torch.isnan(g).all()
 
 
+def test_window_keeps_a_unit_on_the_device_between_open_and_close(cuda, oracle):
+    """One large copy in, many small in-place steps, one large copy out: results equal the oracle's,
+    the host arrays stay untouched until the close, and misuse is refused."""
+    from flextrain_amd import FlexTrainCPUAdam, _C
+    n, shares = 1_000_000, 8
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 16, **HP)
+    p, m, v = _host_state(n, seed=31)
+    before = p.clone()
+    g = (torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16)
+    h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    want = _oracle(oracle, p, g, m, v, 4, torch.bfloat16)
+    token = eng.open_window(p, m, v)
+    per = n // shares
+    for k in range(shares):
+        sl = slice(k * per, (k + 1) * per)
+        eng._step({"step": 4}, h[sl], p[sl], g[sl], m[sl], v[sl], blocking=False)
+    eng.stream_wait()
+    torch.cuda.synchronize()
+    assert torch.equal(p, before)  # nothing has come back yet
+    assert np.array_equal(half_bits(h), want[3])  # but the kernels have run
+    with pytest.raises(ValueError, match="offset inside the open window"):
+        eng._step({"step": 4}, None, p[8:16], g[8:16], m[8:16], v[0:8], blocking=False)
+    sp, sm, sv = _host_state(64, seed=1)
+    small = eng.open_window(sp[:32], sm[:32], sv[:32])
+    with pytest.raises(ValueError, match="inside or entirely outside"):
+        eng._step({"step": 4}, None, sp[16:48], g[16:48], sm[16:48], sv[16:48], blocking=False)
+    eng.close_window(small)
+    with pytest.raises(_C.FtError, match="already belongs"):
+        eng.open_window(p, m, v)
+    eng.close_window(token)
+    eng.synchronize()
+    _assert_equal_bits("window", p, m, v, h, want, torch.bfloat16)
+    with pytest.raises(_C.FtError, match="not open"):
+        eng.close_window(token)
+
+    # windows are reused and grow; a second round on the same memory sees the first one's result
+    p2, m2, v2 = _host_state(2 * n, seed=32)
+    g2 = (torch.randn(2 * n, device=cuda) * 1e-3).to(torch.bfloat16)
+    want2 = _oracle(oracle, p2, g2, m2, v2, 1, None)
+    pn, mn, vn, hn = want
+    oracle.adam_step(pn, to_np(g), mn, vn, step=5, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
+                     weight_decay=HP["weight_decay"], g_dtype=CODE[torch.bfloat16], half_out=hn, half_dtype=CODE[torch.bfloat16])
+    t1, t2 = eng.open_window(p, m, v), eng.open_window(p2, m2, v2)
+    eng._step({"step": 5}, h, p, g, m, v, blocking=False)
+    eng._step({"step": 1}, None, p2, g2, m2, v2, blocking=False)
+    eng.close_window(t2)
+    eng.close_window(t1)
+    eng.synchronize()
+    _assert_equal_bits("window again", p, m, v, h, (pn, mn, vn, hn), torch.bfloat16)
+    _assert_equal_bits("second window", p2, m2, v2, None, want2, None)
+    tokens = [eng.open_window(*_host_state(64, seed=s)) for s in range(4)]
+    with pytest.raises(_C.FtError, match="windows are open"):
+        eng.open_window(*_host_state(64, seed=9))
+    for t in tokens:
+        eng.close_window(t)
+    eng.synchronize()
+
+
+def test_write_through_window(cuda, oracle):
+    """A window whose steps write their results straight to the host arrays: nothing is copied
+    back at the close, the host arrays fill in share by share."""
+    from flextrain_amd import FlexTrainCPUAdam
+    n, shares = 1_000_000, 5
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 16, **HP)
+    p, m, v = _host_state(n, seed=41)
+    before = p.clone()
+    g = (torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16)
+    h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    want = _oracle(oracle, p, g, m, v, 2, torch.bfloat16)
+    token = eng.open_window(p, m, v, write_through=True)
+    per = n // shares
+    for k in range(shares - 1):
+        sl = slice(k * per, (k + 1) * per)
+        eng._step({"step": 2}, h[sl], p[sl], g[sl], m[sl], v[sl], blocking=False)
+    eng.synchronize()
+    done = (shares - 1) * per
+    assert np.array_equal(p.numpy()[:done].view(np.uint32), want[0][:done].view(np.uint32))  # already on the host
+    assert torch.equal(p[done:], before[done:])                                              # not stepped yet
+    eng._step({"step": 2}, h[done:], p[done:], g[done:], m[done:], v[done:], blocking=False)
+    eng.close_window(token)
+    eng.synchronize()
+    _assert_equal_bits("write-through window", p, m, v, h, want, torch.bfloat16)
+
+
 def test_config5_offloaded_7b_optimizer(cuda, oracle):
     """The offloaded Llama-7B optimizer at the largest size this machine can pin (all 32 layers +
     embedding + lm_head = 6.74e9 elements need 81 GB of pinned memory; a machine that refuses that
