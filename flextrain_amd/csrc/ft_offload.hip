@@ -10,6 +10,7 @@
 
 #include <chrono>
 #include <deque>
+#include <mutex>
 #include <vector>
 
 #include "ft_internal.hpp"
@@ -80,6 +81,7 @@ constexpr size_t kStagedMinElems = 32u * 1024u * 1024u;
 
 struct Engine {
     uint32_t magic = 0x46544f45;  // "FTOE"
+    std::mutex mu;                // one call at a time per handle; different handles are independent
     int device = 0;
     size_t chunk = 0;
     std::vector<Slot> slots;
@@ -292,6 +294,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
 {
     Engine* e = as_engine(handle);
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     fth::AdamObject o;
     int rc = fth::find_adam(id, &o);
     if (rc != FT_OK) return rc;
@@ -449,6 +452,7 @@ int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_
 {
     Engine* e = as_engine(handle);
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     if (!out_window) return fth::fail(FT_EINVAL, "out_window must not be NULL");
     *out_window = -1;
     if (n == 0 || !host_p || !host_m || !host_v) return fth::fail(FT_EINVAL, "p, m, v must not be NULL and n must be positive");
@@ -533,6 +537,7 @@ int ft_offload_window_close(void* handle, int window)
 {
     Engine* e = as_engine(handle);
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     if (window < 0 || window >= kMaxWindows || !e->windows[window].open)
         return fth::fail(FT_ENOENT, "window %d is not open", window);
     Window& w = e->windows[window];
@@ -567,6 +572,7 @@ int ft_offload_set_mode(void* handle, int mode)
 {
     Engine* e = as_engine(handle);
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     if (mode < FT_OFFLOAD_AUTO || mode > FT_OFFLOAD_STAGED_OUT) return fth::fail(FT_EINVAL, "unknown offload mode %d", mode);
     e->mode = mode;
     return FT_OK;
@@ -576,6 +582,7 @@ int ft_offload_stream_wait(void* handle, void* stream, int what)
 {
     Engine* e = as_engine(handle);
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     if (what != 0 && what != 1) return fth::fail(FT_EINVAL, "what must be 0 (kernels) or 1 (write-back)");
     if (!e->stepped) return FT_OK;
     FT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), what == 0 ? e->ev_kernels : e->ev_end, 0));
@@ -586,6 +593,7 @@ int ft_offload_wait(void* handle)
 {
     Engine* e = as_engine(handle);
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     if (!e->stepped) return FT_OK;
     FT_HIP(hipEventSynchronize(e->ev_end));
     FT_HIP(hipEventSynchronize(e->ev_kernels));
@@ -599,6 +607,7 @@ int ft_offload_elapsed_ms(void* handle, float* out_ms)
 {
     Engine* e = as_engine(handle);
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     if (!out_ms) return fth::fail(FT_EINVAL, "out_ms must not be NULL");
     if (!e->stepped) return fth::fail(FT_EINVAL, "no step has been enqueued on this handle");
     FT_HIP(hipEventSynchronize(e->ev_end));
