@@ -28,7 +28,7 @@ N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 8
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
 # profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_699_000, "cfg3": 5_666_695_000, "cfg4": 23_958_258_000, "accumulate": 2_453_897_000}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_664_000, "cfg3": 5_666_695_000, "cfg4": 23_958_237_000, "accumulate": 2_453_897_000}
 
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
 
@@ -226,7 +226,7 @@ def bench_offload(args, torch, dev) -> int:
             "frac_of_bidirectional": 2 * one_way / link["both"],
             "bytes_each_way": n * 12, "device_time_ms": sum(devs) / len(devs) * 1e3,
         },
-        "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_vec_kernel per chunk",
+        "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_tile_kernel per chunk",
                      "achieved": 2 * one_way, "peak": link["both"], "unit": "GB/s", "frac": 2 * one_way / link["both"],
                      "traffic": None},
         "setup": {"pinned_alloc_s": t_alloc, "init_s": t_init, "pinned_gb": 3 * n * 4 / 1e9},
@@ -372,7 +372,7 @@ def bench_pipeline(args, torch, dev) -> int:
                  "measured_bidirectional_gbps": link["both"], "achieved_each_way_gbps": one_way,
                  "achieved_total_gbps": 2 * one_way, "frac_of_unidirectional": one_way / min(link["h2d"], link["d2h"]),
                  "frac_of_bidirectional": 2 * one_way / link["both"]},
-        "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_vec_kernel per share",
+        "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_tile_kernel per share",
                      "achieved": 2 * one_way, "peak": link["both"], "unit": "GB/s", "frac": 2 * one_way / link["both"],
                      "traffic": None},
     }), flush=True)
@@ -503,7 +503,7 @@ def main() -> int:
         "hbm_gbps": achieved,
         "hbm_frac_of_peak": achieved / HBM_PEAK_GBPS,
         "roofline": {
-            "bound": "hbm", "kernel": "adam_vec_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "bound": "hbm", "kernel": "adam_tile_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES[args.workload],
             "algorithmic_bytes_per_launch": alg_bytes, "kernel_ms_avg": upd_avg, "kernel_ms_min": min(upd_ms),
             "kernel_ms_p20_80": percentile_mean(upd_ms),

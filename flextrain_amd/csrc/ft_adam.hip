@@ -17,21 +17,9 @@
 #include "ft_kernels.hpp"
 
 // Launch shape of the update kernel, from sweeps on MI355X at 2e8 elements: one 64-lane wavefront
-// per workgroup, one 4-element unit per lane, one workgroup per tile, non-temporal loads and
+// per workgroup, one 4-element unit per lane, one workgroup per tile, non-temporal loads, streaming
 // stores, and at most 11 workgroups resident per compute unit. More resident wavefronts put more
 // requests in flight than HBM can serve in order and cost up to 8 % of the bandwidth.
-#ifndef FT_ADAM_BLOCK
-#define FT_ADAM_BLOCK 64
-#endif
-#ifndef FT_ADAM_UNROLL
-#define FT_ADAM_UNROLL 1
-#endif
-#ifndef FT_ADAM_NT_LD
-#define FT_ADAM_NT_LD true
-#endif
-#ifndef FT_ADAM_NT_ST
-#define FT_ADAM_NT_ST true
-#endif
 #ifndef FT_ADAM_WAVES_PER_CU
 #define FT_ADAM_WAVES_PER_CU 11
 #endif
@@ -182,8 +170,10 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
     const bool vec_ok = aligned(mb + head * 4, 16) && aligned(vb + head * 4, 16) &&
                         aligned(gb + head * gsz, gsz * 4) && (h == nullptr || aligned(hb + head * 2, 8)) &&
                         aligned(out.p + head, 16) && aligned(out.m + head, 16) && aligned(out.v + head, 16);
-    const size_t nvec = vec_ok ? (n - head) / 4 : 0;
-    const size_t body = nvec * 4;
+    // Whole 64-unit tiles go to the tile kernel, everything else (up to 3 head elements and up to
+    // 258 elements behind the last full tile) to the scalar kernel.
+    const size_t ntiles = vec_ok ? (n - head) / 4 / ftk::kWave : 0;
+    const size_t body = ntiles * ftk::kWave * 4;
 
     auto scalar_part = [&](size_t off, size_t cnt) -> int {
         if (cnt == 0) return FT_OK;
@@ -210,7 +200,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
 
     if (!vec_ok) return scalar_part(0, n);
 
-    if (nvec > 0) {
+    if (ntiles > 0) {
         ftk::AdamArgs a;
         a.p = p + head;
         a.g = gb + head * gsz;
@@ -221,16 +211,20 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.v_out = out.v + head;
         a.h = h ? hb + head * 2 : nullptr;
         a.ctl = ctl;
-        a.n = nvec;
+        a.n = ntiles * ftk::kWave;
         a.c = c;
-        constexpr size_t kTile = static_cast<size_t>(FT_ADAM_BLOCK) * FT_ADAM_UNROLL;
-        size_t blocks = (nvec + kTile - 1) / kTile;  // one tile per workgroup ...
-        const size_t cap = 0x7fffffffu;              // ... unless the grid would overflow
-        if (blocks > cap) blocks = cap;
-        hipLaunchKernelGGL(
-            (ftk::adam_vec_kernel<GT, HT, FT_ADAM_BLOCK, FT_ADAM_UNROLL, FT_ADAM_NT_LD, FT_ADAM_NT_ST>),
-            dim3(static_cast<unsigned>(blocks)), dim3(FT_ADAM_BLOCK), throttle_lds_bytes(48 + 4 * static_cast<unsigned>(gsz)), stream, a);
-        FT_HIP(hipGetLastError());
+        const unsigned lds = throttle_lds_bytes(48 + 4 * static_cast<unsigned>(gsz));
+        const size_t max_grid = 0x7fffffffu;  // one workgroup per tile; a larger count is split
+        for (size_t tile0 = 0; tile0 < ntiles; tile0 += max_grid) {
+            const size_t blocks = (ntiles - tile0 < max_grid) ? (ntiles - tile0) : max_grid;
+            if (ctl)
+                hipLaunchKernelGGL((ftk::adam_tile_kernel<GT, HT, true>), dim3(static_cast<unsigned>(blocks)),
+                                   dim3(ftk::kWave), lds, stream, a, static_cast<uint64_t>(tile0));
+            else
+                hipLaunchKernelGGL((ftk::adam_tile_kernel<GT, HT, false>), dim3(static_cast<unsigned>(blocks)),
+                                   dim3(ftk::kWave), lds, stream, a, static_cast<uint64_t>(tile0));
+            FT_HIP(hipGetLastError());
+        }
     }
     int rc = scalar_part(0, head);
     if (rc != FT_OK) return rc;

@@ -1,7 +1,7 @@
 // ft_kernels.hpp -- gfx950 device code of the optimizer-step hot path.
 //
 // Two kernels carry the traffic:
-//   adam_vec_kernel   fused unscale/clip multiply + Adam/AdamW + low-precision recast. One pass:
+//   adam_tile_kernel   fused unscale/clip multiply + Adam/AdamW + low-precision recast. One pass:
 //                     reads p, m, v (fp32) and g (fp32/fp16/bf16), writes p, m, v and optionally
 //                     the 16-bit copy. HBM-bound: 28 bytes per element with 16-bit g and copy.
 //   grad_stats_kernel one read of g: inf/nan count and sum of squares (2 or 4 bytes per element).
@@ -152,98 +152,54 @@ __device__ __forceinline__ f32x4 load_g4(const void* g, uint64_t unit)
     }
 }
 
-template <int HT, bool NT>
-__device__ __forceinline__ void store_h4(void* h, uint64_t unit, f32x4 p)
+// The update over whole tiles. One 64-lane workgroup per tile of 64 units (256 elements), one unit
+// per lane, straight-line code: the host launches exactly one workgroup per full tile (tile0 lets
+// it split a grid that would overflow) and sends the remainder through the scalar kernel, so there
+// is no bounds check and no loop between the kernel-argument loads and the first vector load.
+// That matters for a wavefront that lives for about 3 microseconds: with the checks in front, the
+// argument loads came in two dependent rounds and the kernel was 1 % slower.
+// Inputs and outputs are the same arrays for an in-place update; the offloaded step may point the
+// outputs elsewhere (staging buffer -> host memory, or the reverse), hence no __restrict__.
+// HT == -1: no low-precision copy. HAS_CTL: a.ctl is read (wave-uniform: one decision per step);
+// the vector loads are issued first, so a skipped step still reads its inputs, and writes nothing.
+template <int GT, int HT, bool HAS_CTL>
+__global__ __launch_bounds__(kWave) void adam_tile_kernel(AdamArgs a, uint64_t tile0)
 {
+    // The decision is fetched first (two scalar loads that depend on the argument load) but only
+    // looked at once the vector loads below are on their way: the empty asm consumes the loaded
+    // registers, and an early return may not move above it. With the check in front, every
+    // wavefront would start with two dependent round trips before its first vector load.
+    uint32_t skip = 0;
+    float ctl_mult = 0.0f;
+    if constexpr (HAS_CTL) {
+        skip = a.ctl->skip;
+        ctl_mult = a.ctl->grad_mult;
+    }
+    const uint64_t t0 = (tile0 + blockIdx.x) * kWave;  // first unit of the tile: wave-uniform
+    const uint64_t i = t0 + threadIdx.x;
+    f32x4 g = load_g4<GT, true>(a.g, i);
+    f32x4 p = ld<true>(reinterpret_cast<const f32x4*>(a.p) + i);
+    f32x4 m = ld<true>(reinterpret_cast<const f32x4*>(a.m) + i);
+    f32x4 v = ld<true>(reinterpret_cast<const f32x4*>(a.v) + i);
+    AdamConsts c = a.c;
+    if constexpr (HAS_CTL) {
+        asm volatile("" ::"v"(g), "v"(p), "v"(m), "v"(v));
+        if (skip) return;
+        c.grad_mult = ctl_mult;
+    }
+    adam_unit(p, g, m, v, c);
+    const __amdgpu_buffer_rsrc_t rp = tile_rsrc(reinterpret_cast<f32x4*>(a.p_out) + t0, kWave * 16),
+                                 rm = tile_rsrc(reinterpret_cast<f32x4*>(a.m_out) + t0, kWave * 16),
+                                 rv = tile_rsrc(reinterpret_cast<f32x4*>(a.v_out) + t0, kWave * 16);
+    st_stream(rp, threadIdx.x * 16, p);
+    st_stream(rm, threadIdx.x * 16, m);
+    st_stream(rv, threadIdx.x * 16, v);
     if constexpr (HT == FT_F16 || HT == FT_BF16) {
+        const __amdgpu_buffer_rsrc_t rh = tile_rsrc(reinterpret_cast<u32x2*>(a.h) + t0, kWave * 8);
         u32x2 w;
         w.x = pack2<HT>(p.x, p.y);
         w.y = pack2<HT>(p.z, p.w);
-        st<NT>(reinterpret_cast<u32x2*>(h) + unit, w);
-    }
-}
-
-// HT == -1: no low-precision copy.
-template <int GT, int HT, int BLOCK, int UNROLL, bool NT_LD, bool NT_ST>
-__global__ __launch_bounds__(BLOCK) void adam_vec_kernel(AdamArgs a)
-{
-    AdamConsts c = a.c;
-    if (a.ctl) {  // wave-uniform: one decision per step
-        if (a.ctl->skip) return;
-        c.grad_mult = a.ctl->grad_mult;
-    }
-    const uint64_t nvec = a.n;
-    constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
-    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
-    // Inputs and outputs are the same arrays for an in-place update; the offloaded step may point
-    // the outputs elsewhere (staging buffer -> host memory, or the reverse), hence no __restrict__.
-    const f32x4* P = reinterpret_cast<const f32x4*>(a.p);
-    const f32x4* M = reinterpret_cast<const f32x4*>(a.m);
-    const f32x4* V = reinterpret_cast<const f32x4*>(a.v);
-    f32x4* PO = reinterpret_cast<f32x4*>(a.p_out);
-    f32x4* MO = reinterpret_cast<f32x4*>(a.m_out);
-    f32x4* VO = reinterpret_cast<f32x4*>(a.v_out);
-
-    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const uint64_t base = tile * kTile + threadIdx.x;
-        f32x4 p[UNROLL], m[UNROLL], v[UNROLL], g[UNROLL];
-        if ((tile + 1) * kTile <= nvec) {
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint64_t i = base + (uint64_t)u * BLOCK;
-                g[u] = load_g4<GT, NT_LD>(a.g, i);
-                p[u] = ld<NT_LD>(P + i);
-                m[u] = ld<NT_LD>(M + i);
-                v[u] = ld<NT_LD>(V + i);
-            }
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) {
-                adam_unit(p[u], g[u], m[u], v[u], c);
-            }
-            if constexpr (NT_ST) {
-                const uint64_t t0 = tile * kTile;  // first unit of the tile: wave-uniform
-                const __amdgpu_buffer_rsrc_t rp = tile_rsrc(PO + t0, kTile * 16), rm = tile_rsrc(MO + t0, kTile * 16),
-                                             rv = tile_rsrc(VO + t0, kTile * 16);
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    const uint32_t lane_unit = threadIdx.x + (uint32_t)u * BLOCK;
-                    st_stream(rp, lane_unit * 16, p[u]);
-                    st_stream(rm, lane_unit * 16, m[u]);
-                    st_stream(rv, lane_unit * 16, v[u]);
-                }
-                if constexpr (HT == FT_F16 || HT == FT_BF16) {
-                    const __amdgpu_buffer_rsrc_t rh = tile_rsrc(reinterpret_cast<u32x2*>(a.h) + t0, kTile * 8);
-#pragma unroll
-                    for (int u = 0; u < UNROLL; ++u) {
-                        u32x2 w;
-                        w.x = pack2<HT>(p[u].x, p[u].y);
-                        w.y = pack2<HT>(p[u].z, p[u].w);
-                        st_stream(rh, (threadIdx.x + (uint32_t)u * BLOCK) * 8, w);
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) {
-                    const uint64_t i = base + (uint64_t)u * BLOCK;
-                    PO[i] = p[u];
-                    MO[i] = m[u];
-                    VO[i] = v[u];
-                    store_h4<HT, false>(a.h, i, p[u]);
-                }
-            }
-        } else {  // last, partial tile
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint64_t i = base + (uint64_t)u * BLOCK;
-                if (i >= nvec) break;
-                f32x4 gg = load_g4<GT, false>(a.g, i);
-                f32x4 pp = P[i], mm = M[i], vv = V[i];
-                adam_unit(pp, gg, mm, vv, c);
-                PO[i] = pp;
-                MO[i] = mm;
-                VO[i] = vv;
-                store_h4<HT, false>(a.h, i, pp);
-            }
-        }
+        st_stream(rh, threadIdx.x * 8, w);
     }
 }
 
