@@ -17,7 +17,7 @@ Contents
   cases                           JSON list describing every case (step, mode, wd, bias_correction, lr ...)
   tail_<n>_{p,m,v,h}              outputs for n in TAIL_SIZES on the first n shared inputs (AdamW, t=7)
   cfg1_digest                     sha256 of p|m|v after each of 10 AdamW steps on 2^20 elements
-                                  (BASELINE config 1: p~N(0,0.02), fresh g~N(0,1e-3) per step, m=v=0 at t=1)
+                                  (the CPU-runnable configuration: p~N(0,0.02), fresh g~N(0,1e-3) per step, m=v=0 at t=1)
   repeat_same_step_equal          1 if calling the same step twice from identical state copies gave
                                   identical outputs (the cached-power branch of IncrementStep)
 """
@@ -106,7 +106,7 @@ def main():
         oid += 1
         out[f"tail_{n}_p"], out[f"tail_{n}_m"], out[f"tail_{n}_v"], out[f"tail_{n}_h"] = rp, rm, rv, rh
 
-    # BASELINE config 1 at its real size, kept as digests
+    # the CPU-runnable configuration at its real size, kept as digests
     n1 = 1 << 20
     rng = np.random.default_rng(0)
     tp = torch.from_numpy(rng.normal(0, 0.02, n1).astype(np.float32))

@@ -65,7 +65,7 @@ def test_golden_tails(oracle, golden):
 
 
 def test_golden_config1_trajectory(oracle, golden):
-    """BASELINE config 1 at its real size: 2^20 elements, 10 AdamW steps, digests of p|m|v."""
+    """The CPU-runnable configuration at its real size: 2^20 elements, 10 AdamW steps, digests of p|m|v."""
     want = json.loads(bytes(golden["cfg1_digest"]).decode())
     n = 1 << 20
     rng = np.random.default_rng(0)
