@@ -245,6 +245,8 @@ class FlexTrainOptsCoordinator:
         share, so there is no ``.0`` file, as for any empty share in the reference). Waits for the
         steps in flight first. Returns the paths."""
         from .state_files import BACKWARD_SHARE, write_unit_opts
+        if self._open_windows:
+            raise RuntimeError("units %s are being stepped on the GPU; save after clear_backward_pipeline()" % sorted(self._open_windows))
         self.synchronize()
         paths = []
         for u in range(self._num_units):
@@ -258,6 +260,8 @@ class FlexTrainOptsCoordinator:
         the master parameters into the units' low-precision parameters (what the update's copy-out
         would have left there). Group step counters are the caller's to restore."""
         from .state_files import BACKWARD_SHARE, read_unit_opts
+        if self._open_windows:
+            raise RuntimeError("units %s are being stepped on the GPU; load after clear_backward_pipeline()" % sorted(self._open_windows))
         self.synchronize()
         for u in range(self._num_units):
             if self._offload:
