@@ -30,7 +30,7 @@
 #define FT_STATS_UNROLL 4
 #endif
 #ifndef FT_STATS_BLOCKS_PER_CU
-#define FT_STATS_BLOCKS_PER_CU 4
+#define FT_STATS_BLOCKS_PER_CU 3
 #endif
 
 namespace {
