@@ -102,3 +102,64 @@ def test_unit_segments_and_gradacc_dtype(cuda):
     opt.update_states()
     opt.step()
     assert not opt._device_acc_grad.any()
+
+
+@pytest.mark.parametrize("offload", [False, True])
+def test_training_loop_with_autograd(cuda, offload):
+    """A small fp16 network trained end to end the way a user would: autograd fills the gradients
+    of parameters that live in the optimizer's flat buffer, the loss is scaled by a dynamic scaler,
+    the optimizer unscales, checks, clips and steps. The loss must fall like that of an fp32
+    torch.optim.AdamW twin fed the same batches, and an injected overflow must cost exactly one
+    skipped step and a halved scale."""
+    from flextrain_amd import FlexTrainAdam
+    from flextrain_amd.loss_scaler import DynamicLossScaler
+    torch.manual_seed(3)
+    d_in, d_hid = 32, 64
+    w1 = torch.nn.Parameter((torch.randn(d_in, d_hid, device=cuda) * 0.2).half())
+    b1 = torch.nn.Parameter(torch.zeros(d_hid, device=cuda).half())
+    w2 = torch.nn.Parameter((torch.randn(d_hid, 1, device=cuda) * 0.2).half())
+    twin = [torch.nn.Parameter(p.detach().float().clone()) for p in (w1, b1, w2)]
+    ref = torch.optim.AdamW([{"params": [twin[0], twin[2]], "weight_decay": 0.01}, {"params": [twin[1]], "weight_decay": 0.0}],
+                            lr=3e-3)
+    scaler = DynamicLossScaler(init_scale=2.0 ** 12, delayed_shift=1, scale_window=10_000)
+    opt = FlexTrainAdam([{"params": [w1, w2], "weight_decay": 0.01}, {"params": [b1], "weight_decay": 0.0}], lr=3e-3,
+                        loss_scaler=scaler, max_grad_norm=10.0, offload=offload)
+
+    def forward(params, x):
+        a, b, c = params
+        return (torch.tanh(x @ a + b) @ c).squeeze(-1)
+
+    target_w = torch.randn(d_in, device=cuda)
+    losses, ref_losses, skipped = [], [], 0
+    for it in range(60):
+        x = torch.randn(256, d_in, device=cuda)
+        y = torch.sin(x @ target_w)
+        loss = ((forward((w1, b1, w2), x.half()).float() - y) ** 2).mean()
+        opt.update_states()
+        scaler.backward(loss)
+        if it == 20:
+            w1.grad[0, 0] = float("inf")  # what an fp16 overflow in backward looks like
+        stepped = opt.step()
+        if not stepped:
+            skipped += 1
+            for g in opt.param_groups:  # a skipped step does not count (the caller's policy)
+                g["step"] -= 1
+        losses.append(float(loss.detach()))
+        ref_loss = ((forward(twin, x) - y) ** 2).mean()
+        ref.zero_grad()
+        ref_loss.backward()
+        if it != 20:
+            ref.step()
+        ref_losses.append(float(ref_loss.detach()))
+    assert skipped == 1 and scaler.loss_scale == 2.0 ** 11
+    assert opt.param_groups[0]["step"] == 59
+    first, last = sum(losses[:5]) / 5, sum(losses[-5:]) / 5
+    ref_last = sum(ref_losses[-5:]) / 5
+    print(f"[training loop offload={offload}] loss {first:.4f} -> {last:.4f} (fp32 twin {ref_last:.4f})", flush=True)
+    assert last < 0.6 * first
+    assert abs(last - ref_last) <= 0.1 * ref_last + 5e-3
+    # parameters are the fp16 rounding of the master copy, and close to the fp32 twin's
+    master = opt._master_para.to(cuda)
+    assert torch.equal(opt._device_para, master.half())
+    flat_twin = torch.cat([twin[0].detach().reshape(-1), twin[2].detach().reshape(-1), twin[1].detach().reshape(-1)])
+    assert (master - flat_twin).abs().max() < 0.05
