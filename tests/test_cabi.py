@@ -77,3 +77,24 @@ def test_python_surface_fails_loudly_without_the_library(monkeypatch, tmp_path):
     monkeypatch.setattr(_C, "LIB_PATH", str(tmp_path / "libftadam.so"))
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _C.lib()
+
+
+def test_product_code_never_touches_the_checker():
+    """The CPU checker is test infrastructure: nothing in the shipped package may import, load or
+    link it, and the shared library must not depend on it."""
+    import pathlib
+    import re
+    import subprocess
+    root = pathlib.Path(__file__).resolve().parent.parent
+    pattern = re.compile(r"\boracle\b|ftoracle|ft_oracle")
+    offenders = []
+    for path in (root / "flextrain_amd").rglob("*"):
+        if path.suffix in {".py", ".hip", ".hpp", ".h", ".cpp"}:
+            for lineno, line in enumerate(path.read_text().splitlines(), 1):
+                if pattern.search(line):
+                    offenders.append(f"{path.relative_to(root)}:{lineno}: {line.strip()}")
+    assert not offenders, offenders
+    lib = root / "flextrain_amd" / "libftadam.so"
+    if lib.exists():
+        needed = subprocess.run(["readelf", "-d", str(lib)], capture_output=True, text=True).stdout
+        assert "ftoracle" not in needed
