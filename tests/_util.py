@@ -79,6 +79,12 @@ def max_ulp_gpu(dev: torch.Tensor, host: np.ndarray, chunk: int = 1 << 26) -> in
     """Largest ULP distance between a GPU tensor (fp32, or fp16/bf16) and host data of the same
     format (float32 array, or uint16 bit patterns), evaluated on the GPU chunk by chunk. NaN
     against NaN counts as equal, NaN against a number as a huge distance."""
+    return ulp_histogram_gpu(dev, host, chunk)["max"]
+
+
+def ulp_histogram_gpu(dev: torch.Tensor, host: np.ndarray, chunk: int = 1 << 26) -> dict:
+    """How many elements of a GPU tensor lie 0, 1, 2 and more than 2 ULP from host data of the
+    same format, plus the largest distance (see max_ulp_gpu for the conventions)."""
     n = dev.numel()
     assert host.shape[0] == n
     if dev.dtype == torch.float32:
@@ -91,6 +97,7 @@ def max_ulp_gpu(dev: torch.Tensor, host: np.ndarray, chunk: int = 1 << 26) -> in
         raise TypeError(dev.dtype)
     mag = (1 << (width - 1)) - 1
     worst = 0
+    counts = [0, 0, 0, 0]
     for lo in range(0, n, chunk):
         hi = min(n, lo + chunk)
         a = dev[lo:hi].view(idt).to(torch.int64)
@@ -103,4 +110,6 @@ def max_ulp_gpu(dev: torch.Tensor, host: np.ndarray, chunk: int = 1 << 26) -> in
         d = torch.where(a_nan & b_nan, torch.zeros_like(d), d)
         d = torch.where(a_nan ^ b_nan, torch.full_like(d, 1 << 40), d)
         worst = max(worst, int(d.max().item()))
-    return worst
+        exact, one, two = int((d == 0).sum()), int((d == 1).sum()), int((d == 2).sum())
+        counts = [counts[0] + exact, counts[1] + one, counts[2] + two, counts[3] + (hi - lo) - exact - one - two]
+    return {"0": counts[0], "1": counts[1], "2": counts[2], ">2": counts[3], "max": worst}

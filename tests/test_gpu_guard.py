@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import CODE, F16, HALF_ULP, MASTER_ULP, NORM_RTOL, half_bits, max_ulp_gpu, to_np
+from _util import CODE, F16, HALF_ULP, MASTER_ULP, NORM_RTOL, half_bits, max_ulp_gpu, to_np, ulp_histogram_gpu
 
 pytestmark = pytest.mark.gpu
 
@@ -102,8 +102,10 @@ def _apply_oracle(oracle, pn, mn, vn, g, t, grad_mult, half_dtype):
 
 
 def _check_state(tag, p, m, v, h, pn, mn, vn, hn):
-    worst = dict(p=max_ulp_gpu(p, pn), m=max_ulp_gpu(m, mn), v=max_ulp_gpu(v, vn), h=max_ulp_gpu(h, hn))
-    print(f"[{tag}] worst ULP distance: {worst}", flush=True)
+    hist = dict(p=ulp_histogram_gpu(p, pn), m=ulp_histogram_gpu(m, mn), v=ulp_histogram_gpu(v, vn), h=ulp_histogram_gpu(h, hn))
+    worst = {k: x["max"] for k, x in hist.items()}
+    print(f"[{tag}] ULP distance histograms (elements at 0 / 1 / 2 / more): "
+          + "; ".join(f"{k}: {x['0']} / {x['1']} / {x['2']} / {x['>2']}" for k, x in hist.items()), flush=True)
     assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst["h"] <= HALF_ULP, (tag, worst)
 
 
