@@ -77,6 +77,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             FlexTrainCPUAdam.optimizer_id += 1
         self.adam_w_mode = adamw_mode
         self._lib = _C.lib()  # raises if the native library is missing: there is no fallback
+        self._window_tensors = {}  # window token -> the host tensors it mirrors (kept alive while open)
         self._offload_chunk = int(offload_chunk_elems)
         self._offload_slots = int(offload_slots)
         self._offload_mode = int(offload_mode)  # FT_OFFLOAD_* of include/ft_adam.h; 0 = automatic
@@ -213,13 +214,13 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             self._offload_engine(), full_parameter.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n,
             int(bool(write_through)), ctypes.byref(token)))
         # the engine holds raw addresses: keep the tensors alive until the write-back is enqueued
-        self.__dict__.setdefault("_window_tensors", {})[int(token.value)] = (full_parameter, exp_avg, exp_avg_sq)
+        self._window_tensors[int(token.value)] = (full_parameter, exp_avg, exp_avg_sq)
         return int(token.value)
 
     def close_window(self, token: int) -> None:
         """Enqueues the write-back of a window opened with ``open_window`` and returns."""
         _C.check("ft_offload_window_close", self._lib.ft_offload_window_close(self._offload_engine(), int(token)))
-        self.__dict__.get("_window_tensors", {}).pop(int(token), None)
+        self._window_tensors.pop(int(token), None)
 
     def synchronize(self):
         """Waits for every offloaded step enqueued so far (no-op if none was)."""

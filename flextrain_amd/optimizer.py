@@ -84,7 +84,7 @@ class FlexTrainCPUOptimizer(ABC):
             live = [ctx.gradient for ctx in step_contexts if ctx.gradient.numel()]
             if live:
                 from .loss_scaler import GradientGuard  # local import: keeps module load light
-                guard = self.__dict__.get("_step_guard")
+                guard = getattr(self, "_step_guard", None)
                 if guard is None or guard.device != live[0].device:
                     guard = self._step_guard = GradientGuard(live[0].device)
                 guard.begin()
