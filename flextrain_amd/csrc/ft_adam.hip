@@ -9,6 +9,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <cmath>
 #include <mutex>
 #include <unordered_map>
@@ -44,7 +45,7 @@ std::unordered_map<int, void*> g_stats_ws;    // device -> library-owned statist
 std::unordered_map<int, size_t> g_stats_ws_bytes;
 int g_adam_waves_per_cu = FT_ADAM_WAVES_PER_CU;
 std::unordered_map<int, int> g_lds_per_cu;   // device -> bytes of LDS per compute unit
-int g_stats_blocks_per_cu = FT_STATS_BLOCKS_PER_CU;
+std::atomic<int> g_stats_blocks_per_cu{FT_STATS_BLOCKS_PER_CU};  // read without the lock
 
 constexpr int kMaxStatsBlocks = 8192;
 
@@ -463,7 +464,7 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
     if (nvec > 0) {
         constexpr size_t kTile = static_cast<size_t>(FT_STATS_BLOCK) * FT_STATS_UNROLL;
         size_t b = (nvec + kTile - 1) / kTile;
-        size_t cap = static_cast<size_t>(fth::cu_count()) * static_cast<size_t>(g_stats_blocks_per_cu);
+        size_t cap = static_cast<size_t>(fth::cu_count()) * static_cast<size_t>(g_stats_blocks_per_cu.load());
         if (cap > static_cast<size_t>(kMaxStatsBlocks)) cap = kMaxStatsBlocks;
         if (b > cap) b = cap;
         blocks = static_cast<int>(b);
