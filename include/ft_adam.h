@@ -142,7 +142,9 @@ int ft_pinned_free(void* ptr);
  * (+ the low-precision copy when it lives on the host) on a third, ordered per buffer slot by
  * events, never by a device-wide wait.
  *
- * ft_offload_create: chunk_elems elements per chunk, n_slots (>= 2) device buffer sets.
+ * ft_offload_create: chunk_elems elements per chunk, n_slots (>= 2) device buffer sets. A step of
+ *                    more than 96 chunks makes the engine grow its chunk (and its buffers) so that
+ *                    96 suffice: longer bursts of copies run markedly slower on this platform.
  * ft_offload_step:   enqueues one full step over n elements and returns; host_p/m/v are pinned
  *                    host arrays; g and half_out are device pointers when *_on_host == 0 and
  *                    pinned host pointers otherwise (half_out may be NULL). The step starts

@@ -324,6 +324,22 @@ def test_write_through_window(cuda, oracle):
     _assert_equal_bits("write-through window", p, m, v, h, want, torch.bfloat16)
 
 
+@pytest.mark.parametrize("mode", [1, 3, 4])
+def test_engine_grows_its_chunk_for_long_steps(cuda, oracle, mode):
+    """A step that would need more than 96 chunks makes the engine enlarge its chunk first (long
+    bursts of copies run slowly); results are unaffected, also for the steps that follow."""
+    from flextrain_amd import FlexTrainCPUAdam
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 12, offload_slots=2, offload_mode=mode, **HP)
+    h = None
+    for n, t in ((300_000, 1), (1_000_003, 2), (5_000, 3), (2_500_000, 4)):  # 74, then 245 (grows), 1, 3 chunks
+        p, m, v = _host_state(n, seed=60 + t)
+        g = (torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16)
+        h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+        want = _oracle(oracle, p, g, m, v, t, torch.bfloat16)
+        eng._step({"step": t}, h, p, g, m, v)
+        _assert_equal_bits(f"grown chunk mode={mode} n={n}", p, m, v, h, want, torch.bfloat16)
+
+
 def test_config5_offloaded_7b_optimizer(cuda, oracle):
     """The offloaded Llama-7B optimizer at the largest size this machine can pin (all 32 layers +
     embedding + lm_head = 6.74e9 elements need 81 GB of pinned memory; a machine that refuses that
