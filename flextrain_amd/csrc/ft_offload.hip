@@ -98,6 +98,7 @@ struct Engine {
     bool stepped = false;
     size_t cursor = 0;  // chunks enqueued so far; slots are taken round-robin across steps
     int mode = FT_OFFLOAD_AUTO;
+    size_t burst_chunks = 0;  // staged chunks enqueued since the pipeline was last seen idle
     std::deque<Pending> recent;        // steps whose write-back may still be in flight, oldest first
     std::vector<hipEvent_t> free_events;
     Window windows[kMaxWindows];
@@ -408,8 +409,19 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
 
     // How the state crosses the link (see ft_offload_set_mode). Staged = SDMA copy through a device
     // buffer slot; direct = the update kernel itself reads or writes the pinned host arrays.
+    // Automatic: staged for large steps, but only while the burst of chunks enqueued since the
+    // pipeline was last idle stays short (see kMaxChunksPerStep: the same limit holds across calls;
+    // 24 units x 4 staged steps run at 49 GB/s each way, x 6 at 25 GB/s); direct otherwise.
     int mode = e->mode;
-    if (mode == FT_OFFLOAD_AUTO) mode = (n >= kStagedMinElems) ? FT_OFFLOAD_STAGED : FT_OFFLOAD_DIRECT;
+    if (e->burst_chunks > 0 && hipStreamQuery(e->s_d2h) == hipSuccess && hipStreamQuery(e->s_k) == hipSuccess &&
+        hipStreamQuery(e->s_h2d) == hipSuccess)
+        e->burst_chunks = 0;
+    (void)hipGetLastError();  // hipErrorNotReady from the queries is not an error
+    if (mode == FT_OFFLOAD_AUTO) {
+        const size_t chunks = (n + e->chunk - 1) / e->chunk;
+        const bool fits = chunks > kMaxChunksPerStep || e->burst_chunks + chunks <= kMaxChunksPerStep;
+        mode = (n >= kStagedMinElems && fits) ? FT_OFFLOAD_STAGED : FT_OFFLOAD_DIRECT;
+    }
     const bool in_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_IN;
     const bool out_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_OUT;
     const bool stage_g = g_on_host && in_staged;
@@ -433,6 +445,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
         void* kh = half_out ? static_cast<void*>(hb + off * 2) : nullptr;
         Slot* slot = nullptr;
         if (in_staged || out_staged) {
+            ++e->burst_chunks;
             // Round-robin over all steps, not per step: a step that is a single chunk (one share
             // of a unit) must not queue behind the previous step's last use of the same slot.
             slot = &e->slots[e->cursor++ % e->slots.size()];
@@ -638,6 +651,7 @@ int ft_offload_wait(void* handle)
     // everything enqueued so far has finished: nothing is pending any more
     for (Pending& pd : e->recent) e->free_events.push_back(pd.done);
     e->recent.clear();
+    e->burst_chunks = 0;
     return FT_OK;
 }
 
