@@ -320,7 +320,8 @@ def bench_pipeline(args, torch, dev) -> int:
         opt.cpu_optimizer._offload_slots = args.slots
         try:
             coord = FlexTrainOptsCoordinator()
-            coord.initialize(opt, flat, mb, offload=True, unit_windows=args.windows != "off",
+            coord.initialize(opt, flat, mb, offload=True,
+                             unit_windows={"auto": None, "off": False}.get(args.windows, True),
                              window_write_through=args.windows == "write_through")
         except _C.FtError:
             coord = None
@@ -386,7 +387,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate"])
     ap.add_argument("--micro-batches", type=int, default=4, help="pipeline: shares per unit")
-    ap.add_argument("--windows", default="off", choices=["off", "write_through", "copy_back"],
+    ap.add_argument("--windows", default="auto", choices=["auto", "off", "write_through", "copy_back"],
                     help="pipeline: keep a whole unit's state on the GPU while it is stepped (prefetched one unit ahead)")
     ap.add_argument("--chunk-elems", type=int, default=64 * 1024 * 1024, help="cfg5: elements per streamed chunk")
     ap.add_argument("--slots", type=int, default=3, help="cfg5: device buffer sets of the pipeline")

@@ -45,18 +45,16 @@ struct Pending {
 constexpr size_t kMaxPending = 8;
 
 // A window keeps the whole state of one unit on the device between ft_offload_window_open and
-// ft_offload_window_close: one large H2D per array when it opens (in pieces, each with its own
-// event, so that a step on the front of the unit need not wait for the back), any number of steps
-// on sub-ranges that run as plain kernels on the device copy, and the way back either as one large
-// D2H per array when it closes or -- write_through -- by the step kernels themselves, which then
-// write their results straight to the host arrays (each element may then be stepped once per
-// window). Measured on the 24-layer schedule with 16 shares per unit (each way, concurrently):
-// per-share direct 43.5 GB/s; write-through windows 44.5 GB/s, every iteration alike; copy-back
-// windows 47.7 GB/s in most iterations but 28 GB/s in about one of six, when copies that were
-// enqueued long before their dependencies resolved end up queued behind one another on one copy
-// engine (waiting on the host until a copy can start removes those iterations, at the price of a
-// host-device synchronisation per unit, which a training loop cannot afford).
-constexpr size_t kWindowPieceElems = 64u * 1024u * 1024u;  // about 256 MiB per array and copy
+// ft_offload_window_close: one large H2D per array when it opens (in pieces of up to 1 GiB, each
+// with its own event), any number of steps on sub-ranges that run as plain kernels on the device
+// copy, and the way back either as one large D2H per array when it closes or -- write_through -- by
+// the step kernels themselves, which then write their results straight to the host arrays (each
+// element may then be stepped once per window). Measured on the 24-layer schedule with 16 shares
+// per unit (each way, concurrently): per-share direct 43.4 GB/s; write-through windows 43.7 GB/s;
+// copy-back windows 47.2 GB/s, every iteration alike. Few, large copies matter: with 256 MiB pieces
+// (24 copies per unit, 576 per iteration) one iteration in six ran at half speed, the same
+// degradation of long bursts of copies that kMaxChunksPerStep guards against.
+constexpr size_t kWindowPieceElems = 256u * 1024u * 1024u;  // about 1 GiB per array and copy
 constexpr int kMaxWindows = 4;
 
 struct Window {

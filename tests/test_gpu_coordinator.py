@@ -15,7 +15,7 @@ class _Unit:
         self.paras = paras
 
 
-@pytest.mark.parametrize("offload,windows", [(True, "copy_back"), (True, "write_through"), (True, None), (False, None)])
+@pytest.mark.parametrize("offload,windows", [(True, "copy_back"), (True, "write_through"), (True, "off"), (True, "auto"), (False, "off")])
 def test_backward_pipeline_matches_oracle(cuda, oracle, offload, windows):
     from flextrain_amd import FlexTrainAdam
     from flextrain_amd.coordinator import FlexTrainOptsCoordinator
@@ -38,8 +38,10 @@ def test_backward_pipeline_matches_oracle(cuda, oracle, offload, windows):
     assert opt.non_layerwise_numel == 0
     assert [(s.start, s.end) for s in opt.unit_group_segments[0]] == [(0, w_numel), (w_numel, unit_numel)]
     coord = FlexTrainOptsCoordinator()
-    coord.initialize(opt, flat, micro_batches, offload=offload, unit_windows=windows is not None,
+    coord.initialize(opt, flat, micro_batches, offload=offload,
+                     unit_windows={"auto": None, "off": False}.get(windows, True),
                      window_write_through=windows == "write_through")
+    assert coord._unit_windows == (offload and windows != "off")  # small shares: the automatic choice is windows
     assert coord.unit_master_parameter(0).is_pinned() == offload
 
     # oracle state, seeded the same way
