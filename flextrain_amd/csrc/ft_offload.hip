@@ -94,6 +94,7 @@ struct Engine {
     hipEvent_t ev_end = nullptr;    // last D2H of the last step
     hipEvent_t ev_kernels = nullptr;  // last kernel of the last step
     bool stepped = false;
+    bool end_recorded = false;  // ev_begin / ev_end have been recorded at least once
     size_t cursor = 0;  // chunks enqueued so far; slots are taken round-robin across steps
     int mode = FT_OFFLOAD_AUTO;
     size_t burst_chunks = 0;  // staged chunks enqueued since the pipeline was last seen idle
@@ -380,7 +381,6 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     if (window) {
         const size_t last_piece = (window_off + n - 1) / window->piece;
         FT_HIP(hipStreamWaitEvent(e->s_k, window->piece_done[last_piece], 0));
-        FT_HIP(hipEventRecord(e->ev_begin, e->s_k));
         float* out[3] = {nullptr, nullptr, nullptr};  // nullptr = in place on the device copy
         if (window->write_through) {
             out[0] = static_cast<float*>(host_p);
@@ -391,9 +391,10 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
                               window->dev[2] + window_off, half_out, half_dtype, n,
                               static_cast<const ft_step_control_t*>(ctl), e->s_k, out[0], out[1], out[2]);
         if (rc != FT_OK) return rc;
+        // Only the kernel stream is touched: the copy streams carry the windows' large copies and
+        // nothing else (hundreds of small steps per iteration would otherwise add as many markers
+        // to the D2H stream).
         FT_HIP(hipEventRecord(e->ev_kernels, e->s_k));
-        FT_HIP(hipStreamWaitEvent(e->s_d2h, e->ev_kernels, 0));
-        FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
         e->stepped = true;
         return FT_OK;
     }
@@ -492,6 +493,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     FT_HIP(hipStreamWaitEvent(e->s_d2h, e->ev_kernels, 0));
     FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
     e->stepped = true;
+    e->end_recorded = true;
 
     return remember_writeback(e, mine);
 }
@@ -606,6 +608,7 @@ int ft_offload_window_close(void* handle, int window)
     FT_HIP(hipEventRecord(w.d2h_done, e->s_d2h));
     FT_HIP(hipEventRecord(e->ev_end, e->s_d2h));
     e->stepped = true;
+    e->end_recorded = true;
     for (int a = 0; a < 3; ++a) {
         mine.lo[a] = w.host[a];
         mine.hi[a] = w.host[a] + w.n * 4;
@@ -634,7 +637,10 @@ int ft_offload_stream_wait(void* handle, void* stream, int what)
     std::lock_guard<std::mutex> lock(e->mu);
     if (what != 0 && what != 1) return fth::fail(FT_EINVAL, "what must be 0 (kernels) or 1 (write-back)");
     if (!e->stepped) return FT_OK;
-    FT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), what == 0 ? e->ev_kernels : e->ev_end, 0));
+    // the write-back is over when the D2H stream has passed the last step that used it and the
+    // kernels (which write host memory themselves in the direct and write-through forms) are done
+    if (what == 1 && e->end_recorded) FT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), e->ev_end, 0));
+    FT_HIP(hipStreamWaitEvent(static_cast<hipStream_t>(stream), e->ev_kernels, 0));
     return FT_OK;
 }
 
@@ -644,7 +650,7 @@ int ft_offload_wait(void* handle)
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
     std::lock_guard<std::mutex> lock(e->mu);
     if (!e->stepped) return FT_OK;
-    FT_HIP(hipEventSynchronize(e->ev_end));
+    if (e->end_recorded) FT_HIP(hipEventSynchronize(e->ev_end));
     FT_HIP(hipEventSynchronize(e->ev_kernels));
     // everything enqueued so far has finished: nothing is pending any more
     for (Pending& pd : e->recent) e->free_events.push_back(pd.done);
@@ -659,7 +665,7 @@ int ft_offload_elapsed_ms(void* handle, float* out_ms)
     if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
     std::lock_guard<std::mutex> lock(e->mu);
     if (!out_ms) return fth::fail(FT_EINVAL, "out_ms must not be NULL");
-    if (!e->stepped) return fth::fail(FT_EINVAL, "no step has been enqueued on this handle");
+    if (!e->end_recorded) return fth::fail(FT_EINVAL, "no step that moves data has been enqueued on this handle");
     FT_HIP(hipEventSynchronize(e->ev_end));
     FT_HIP(hipEventElapsedTime(out_ms, e->ev_begin, e->ev_end));
     return FT_OK;

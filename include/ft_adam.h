@@ -156,7 +156,8 @@ int ft_pinned_free(void* ptr);
  *                    half_out read), what == 1 for its write-back to host memory.
  * ft_offload_wait:   blocks the calling thread until everything enqueued so far has finished.
  * ft_offload_elapsed_ms: device time between the first H2D and the last D2H of the last
- *                    enqueued step (waits for it).
+ *                    enqueued step that ran through the pipeline (waits for it; a step inside a
+ *                    window is a bare kernel and leaves this figure alone).
  */
 enum {
     FT_OFFLOAD_AUTO = 0,       /* staged for steps of at least 32 Mi elements, direct for shorter ones */
