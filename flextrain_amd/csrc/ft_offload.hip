@@ -187,11 +187,11 @@ int resize_slots(Engine* e, size_t chunk_elems)
 
 // Orders the H2D and kernel streams behind the newest earlier write-back that touched any of the
 // host ranges in `mine` (the D2H stream is in order, so that one event covers all older ones).
-int wait_for_overlapping_writebacks(Engine* e, const Pending& mine)
+int wait_for_overlapping_writebacks(Engine* e, const Pending& mine, bool h2d_too = true)
 {
     for (auto it = e->recent.rbegin(); it != e->recent.rend(); ++it) {
         if (it->overlaps(mine)) {
-            FT_HIP(hipStreamWaitEvent(e->s_h2d, it->done, 0));
+            if (h2d_too) FT_HIP(hipStreamWaitEvent(e->s_h2d, it->done, 0));
             FT_HIP(hipStreamWaitEvent(e->s_k, it->done, 0));
             break;
         }
@@ -366,15 +366,32 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     add_range(host_v, n * 4);
     if (half_out && half_on_host) add_range(half_out, n * 2);
 
+    // How the state crosses the link (see ft_offload_set_mode). Staged = SDMA copy through a device
+    // buffer slot; direct = the update kernel itself reads or writes the pinned host arrays.
+    // Automatic: staged for large steps, but only while the burst of chunks enqueued since the
+    // pipeline was last idle stays short (see kMaxChunksPerStep: the same limit holds across calls;
+    // 24 units x 4 staged steps run at 49 GB/s each way, x 6 at 25 GB/s); direct otherwise.
+    int mode = e->mode;
+    if (e->burst_chunks > 0 && hipStreamQuery(e->s_d2h) == hipSuccess && hipStreamQuery(e->s_k) == hipSuccess &&
+        hipStreamQuery(e->s_h2d) == hipSuccess)
+        e->burst_chunks = 0;
+    (void)hipGetLastError();  // hipErrorNotReady from the queries is not an error
+    if (mode == FT_OFFLOAD_AUTO) {
+        const size_t chunks = (n + e->chunk - 1) / e->chunk;
+        const bool fits = chunks > kMaxChunksPerStep || e->burst_chunks + chunks <= kMaxChunksPerStep;
+        mode = (n >= kStagedMinElems && fits) ? FT_OFFLOAD_STAGED : FT_OFFLOAD_DIRECT;
+    }
+    const bool in_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_IN;
+    const bool out_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_OUT;
     // The pipeline starts after the producer of g/ctl on the caller's stream ...
-    // (a step inside a window copies nothing, so the H2D stream, which may be prefetching the next
-    // window, is left alone)
+    // (a step that copies nothing in -- inside a window, or with the kernel reading host memory
+    // itself -- leaves the H2D stream alone)
     FT_HIP(hipEventRecord(e->ev_user, user));
-    if (!window) FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_user, 0));
+    if (!window && in_staged) FT_HIP(hipStreamWaitEvent(e->s_h2d, e->ev_user, 0));
     FT_HIP(hipStreamWaitEvent(e->s_k, e->ev_user, 0));
     // ... and after the newest earlier step that wrote to the same host memory (the D2H stream is
     // in order, so that one event covers all older ones).
-    if (!window && (rc = wait_for_overlapping_writebacks(e, mine)) != FT_OK) return rc;
+    if (!window && (rc = wait_for_overlapping_writebacks(e, mine, in_staged)) != FT_OK) return rc;
 
     // State held in an open window: the step is one in-place kernel on the device copy; nothing
     // crosses the link until the window closes.
@@ -398,7 +415,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
         e->stepped = true;
         return FT_OK;
     }
-    FT_HIP(hipEventRecord(e->ev_begin, e->s_h2d));
+    FT_HIP(hipEventRecord(e->ev_begin, in_staged ? e->s_h2d : e->s_k));
 
     float* hp = static_cast<float*>(host_p);
     float* hm = static_cast<float*>(host_m);
@@ -406,23 +423,6 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     const char* gb = static_cast<const char*>(g);
     char* hb = static_cast<char*>(half_out);
 
-    // How the state crosses the link (see ft_offload_set_mode). Staged = SDMA copy through a device
-    // buffer slot; direct = the update kernel itself reads or writes the pinned host arrays.
-    // Automatic: staged for large steps, but only while the burst of chunks enqueued since the
-    // pipeline was last idle stays short (see kMaxChunksPerStep: the same limit holds across calls;
-    // 24 units x 4 staged steps run at 49 GB/s each way, x 6 at 25 GB/s); direct otherwise.
-    int mode = e->mode;
-    if (e->burst_chunks > 0 && hipStreamQuery(e->s_d2h) == hipSuccess && hipStreamQuery(e->s_k) == hipSuccess &&
-        hipStreamQuery(e->s_h2d) == hipSuccess)
-        e->burst_chunks = 0;
-    (void)hipGetLastError();  // hipErrorNotReady from the queries is not an error
-    if (mode == FT_OFFLOAD_AUTO) {
-        const size_t chunks = (n + e->chunk - 1) / e->chunk;
-        const bool fits = chunks > kMaxChunksPerStep || e->burst_chunks + chunks <= kMaxChunksPerStep;
-        mode = (n >= kStagedMinElems && fits) ? FT_OFFLOAD_STAGED : FT_OFFLOAD_DIRECT;
-    }
-    const bool in_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_IN;
-    const bool out_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_OUT;
     const bool stage_g = g_on_host && in_staged;
     const bool stage_h = half_out && half_on_host && out_staged;
     if ((in_staged || out_staged) && (n + e->chunk - 1) / e->chunk > kMaxChunksPerStep) {
