@@ -43,12 +43,16 @@ def percentile_mean(samples, lo=0.2, hi=0.8):
 
 
 def make_inputs(torch, n, g_dtype, g_std, device, scale=1.0):
+    """p, g, m, v and the 16-bit copy of one partition, in the library's own layout for the arrays
+    of an update (one allocation, staggered starts), filled in place from a seeded generator."""
+    from flextrain_amd.memory import allocate_device_arrays
     gen = torch.Generator(device=device).manual_seed(0)
-    p = torch.randn(n, device=device, generator=gen) * 0.02
-    m = torch.randn(n, device=device, generator=gen) * 1e-4
-    v = torch.rand(n, device=device, generator=gen) * 1e-6
-    g = (torch.randn(n, device=device, generator=gen) * (g_std * scale)).to(g_dtype)
-    h = torch.empty(n, dtype=torch.bfloat16, device=device)
+    p, m, v, g, h = allocate_device_arrays(
+        [(n, torch.float32)] * 3 + [(n, g_dtype), (n, torch.bfloat16)], device)
+    p.normal_(0.0, 0.02, generator=gen)
+    m.normal_(0.0, 1e-4, generator=gen)
+    v.uniform_(0.0, 1e-6, generator=gen)
+    g.normal_(0.0, g_std * scale, generator=gen)
     return p, g, m, v, h
 
 
@@ -243,8 +247,9 @@ def bench_accumulate(args, torch, dev) -> int:
     from flextrain_amd.loss_scaler import GradientGuard
     n = N_7B_LAYER
     guard = GradientGuard(dev)
-    acc = torch.zeros(n, device=dev)
-    g = (torch.randn(n, device=dev) * 1e-3).to(torch.bfloat16)
+    from flextrain_amd.memory import allocate_device_arrays
+    acc, g = allocate_device_arrays([(n, torch.float32), (n, torch.bfloat16)], dev)
+    g.normal_(0.0, 1e-3, generator=torch.Generator(device=dev).manual_seed(0))
     if args.calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
         scratch = torch.empty_like(acc)
         for _ in range(3):

@@ -199,6 +199,49 @@ def allocate_memory_chunks(numel: int, chunks: Union[int, Tuple[int, ...]], dtyp
     return allocate_memory(numel * prod(chunks), dtype, device, pin_memory).view(*chunks, numel)
 
 
+_ARENA_ALIGN = 2 * 1024 * 1024
+_ARENA_SKEW = 2 * 1024
+
+
+def device_arena_layout(specs: Sequence[Tuple[int, torch.dtype]]) -> Tuple[List[int], int]:
+    """Byte offsets of the arrays of ``allocate_device_arrays`` inside their one allocation, and
+    its total size. Array k starts at the next 2 MiB boundary plus k x 2 KiB; arrays smaller than
+    2 MiB are only 256-byte aligned."""
+    offsets, cursor = [], 0
+    for k, (numel, dtype) in enumerate(specs):
+        nbytes = numel * dtype.itemsize
+        if nbytes >= _ARENA_ALIGN:
+            cursor = _get_aligned_numel(cursor, _ARENA_ALIGN) + (k * _ARENA_SKEW) % _ARENA_ALIGN
+        else:
+            cursor = _get_aligned_numel(cursor, 256)
+        offsets.append(cursor)
+        cursor += nbytes
+    return offsets, max(cursor, 1)
+
+
+def allocate_device_arrays(specs: Sequence[Tuple[int, torch.dtype]], device) -> List[Tensor]:
+    """Zero-filled flat arrays for one update (parameters, moments, gradients, 16-bit copy ...),
+    carved out of ONE device allocation.
+
+    The update kernel streams all of its arrays at the same element index at once, and how their
+    addresses relate decides how the streams collide in the memory system: arrays that torch
+    happened to place badly have run the kernel 2-3 % slower than the same arrays in one
+    allocation (855 M elements: 82 % against 84-85 % of peak bandwidth). One allocation with
+    2 MiB-aligned starts and a 2 KiB stagger from array to array was the best or within 0.5 % of
+    the best of the layouts measured, at every base address tried. The arrays keep the allocation
+    alive; nothing else about them is special."""
+    global _ALLOCATED_VRAM_SIZE
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise ValueError("allocate_device_arrays is for GPU memory; host state uses pinned_empty / allocate_memory")
+    offsets, total = device_arena_layout(specs)
+    total += _ARENA_ALIGN  # room to start the layout on a 2 MiB boundary wherever torch puts the block
+    _ALLOCATED_VRAM_SIZE += total
+    arena = torch.zeros(total, dtype=torch.uint8, device=device)
+    lead = -arena.data_ptr() % _ARENA_ALIGN
+    return [arena[lead + o:lead + o + numel * dtype.itemsize].view(dtype) for o, (numel, dtype) in zip(offsets, specs)]
+
+
 def get_allocated_dram_size() -> int:
     return _ALLOCATED_DRAM_SIZE
 

@@ -128,10 +128,21 @@ class FlexTrainCPUOptimizer(ABC):
         """
         if not hasattr(self, "_param_group"):
             self._param_group = {STEP_KEY: 0}
-            self._half_parameter = self._allocate(numel, device_dtype, "empty")
-            self._full_parameter = self._allocate(numel, master_dtype, "randn")
-            self._gradient = self._allocate(numel, master_dtype, "randn")
-            self._optimizer_states = self._init_optimizer_states(numel, master_dtype)
+            if self.state_device == "cpu":
+                self._half_parameter = self._allocate(numel, device_dtype, "empty")
+                self._full_parameter = self._allocate(numel, master_dtype, "randn")
+                self._gradient = self._allocate(numel, master_dtype, "randn")
+                self._optimizer_states = self._init_optimizer_states(numel, master_dtype)
+            else:  # resident: all arrays of the update in one allocation with staggered starts
+                from .memory import allocate_device_arrays
+                states = len(self._init_optimizer_states(1, master_dtype))
+                arrays = allocate_device_arrays(
+                    [(numel, device_dtype)] + [(numel, master_dtype)] * (2 + states),
+                    torch.device("cuda", torch.cuda.current_device()))
+                self._half_parameter, self._full_parameter, self._gradient = arrays[:3]
+                self._full_parameter.normal_()
+                self._gradient.normal_()
+                self._optimizer_states = tuple(arrays[3:])
         self._param_group[STEP_KEY] += 1
         self._step(
             self._param_group,

@@ -163,3 +163,50 @@ def test_training_loop_with_autograd(cuda, offload):
     assert torch.equal(opt._device_para, master.half())
     flat_twin = torch.cat([twin[0].detach().reshape(-1), twin[2].detach().reshape(-1), twin[1].detach().reshape(-1)])
     assert (master - flat_twin).abs().max() < 0.05
+
+
+def test_device_arrays_share_one_allocation(cuda):
+    """The arrays of an update come zero-filled out of one allocation, each of the right type and
+    length, 2 MiB-aligned plus a 2 KiB stagger, without overlap; a step on them equals a step on
+    separately allocated tensors bit for bit (placement changes speed, never results)."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.memory import allocate_device_arrays
+    n = (3 << 20) + 5
+    specs = [(n, torch.float32)] * 3 + [(n, torch.bfloat16)] * 2
+    arrays = allocate_device_arrays(specs, cuda)
+    assert [(a.numel(), a.dtype) for a in arrays] == specs
+    assert [a.data_ptr() % (2 << 20) for a in arrays] == [0, 2048, 4096, 6144, 8192]
+    spans = sorted((a.data_ptr(), a.data_ptr() + a.numel() * a.element_size()) for a in arrays)
+    assert all(spans[k][1] <= spans[k + 1][0] for k in range(len(spans) - 1))
+    assert all(not a.any() for a in arrays)
+    p, m, v, g, h = arrays
+    gen = torch.Generator(device=cuda).manual_seed(5)
+    p.normal_(0, 0.02, generator=gen); g.normal_(0, 1e-3, generator=gen)
+    p2, m2, v2, g2, h2 = p.clone(), m.clone(), v.clone(), g.clone(), h.clone()
+    eng = FlexTrainCPUAdam(lr=1e-3, weight_decay=0.01)
+    for t in (1, 2):
+        eng._step({"step": t}, h, p, g, m, v)
+        eng._step({"step": t}, h2, p2, g2, m2, v2)
+    for a, b in ((p, p2), (m, m2), (v, v2), (h, h2)):
+        assert torch.equal(a, b)
+    with pytest.raises(ValueError):
+        allocate_device_arrays(specs, "cpu")
+
+
+@pytest.mark.parametrize("state_device", ["cuda", "cpu"])
+def test_profile_step_runs_on_private_buffers(cuda, state_device):
+    """The reference's own micro-benchmark entry (``flextrain/optimizer.py:71-95``): buffers are
+    made once, every call is one more step, and the parameters move."""
+    from flextrain_amd import FlexTrainCPUAdam
+    eng = FlexTrainCPUAdam(lr=1e-2)
+    eng.state_device = state_device
+    eng.profile_step(1 << 18, torch.bfloat16, torch.float32)
+    first = eng._full_parameter.clone()
+    buffers = (eng._half_parameter.data_ptr(), eng._full_parameter.data_ptr(), eng._gradient.data_ptr())
+    eng.profile_step(1 << 18, torch.bfloat16, torch.float32)
+    eng.synchronize()
+    assert eng._param_group["step"] == 2
+    assert buffers == (eng._half_parameter.data_ptr(), eng._full_parameter.data_ptr(), eng._gradient.data_ptr())
+    assert not torch.equal(first, eng._full_parameter)
+    assert torch.equal(eng._half_parameter.float().cpu(), eng._full_parameter.bfloat16().float().cpu())
+    assert eng._full_parameter.is_cuda == (state_device == "cuda")

@@ -13,6 +13,7 @@ from flextrain_amd.memory import (
     RotateContainer,
     allocate_optimal,
     copy_segments,
+    device_arena_layout,
     get_page_aligned_numel,
     get_page_aligned_padding_numel,
     get_partition_aligned_numel,
@@ -134,3 +135,20 @@ def test_move_into_contiguous_and_para_group():
     assert grads.tolist() == [0, 0, 0, 0, 0, 0, 1, 1]
     group.detach_para()
     assert all(p.numel() == 0 for p in params)
+
+
+def test_device_arena_layout_staggers_large_arrays_and_packs_small_ones():
+    """Arrays of 2 MiB and more start on a 2 MiB boundary plus 2 KiB times their index and never
+    overlap; small ones are only 256-byte aligned; the total covers the last array."""
+    mib2 = 2 * 1024 * 1024
+    specs = [(202_383_360, torch.float32)] * 3 + [(202_383_360, torch.bfloat16)] * 2
+    offsets, total = device_arena_layout(specs)
+    assert [o % mib2 for o in offsets] == [0, 2048, 4096, 6144, 8192]
+    ends = [o + n * dt.itemsize for o, (n, dt) in zip(offsets, specs)]
+    assert all(ends[k] <= offsets[k + 1] for k in range(4)) and total == ends[-1]
+    assert total - sum(n * dt.itemsize for n, dt in specs) < 5 * mib2          # padding is bounded
+
+    offsets, total = device_arena_layout([(7, torch.float32), (3, torch.float16), (1 << 20, torch.float32), (5, torch.float32)])
+    assert offsets[0] == 0 and offsets[1] == 256 and offsets[2] == mib2 + 2 * 2048
+    assert offsets[3] == -(-(offsets[2] + (4 << 20)) // 256) * 256 and total == offsets[3] + 20
+    assert device_arena_layout([]) == ([], 1)
