@@ -158,6 +158,8 @@ void destroy_engine(Engine* e)
 }
 
 // Re-creates the slots' device buffers for `chunk_elems` per chunk. Waits for the pipeline first.
+// If the device has no room for them the slots are left without buffers (and the chunk as it was):
+// the next staged step tries again at that size, direct steps and windows are not affected.
 int resize_slots(Engine* e, size_t chunk_elems)
 {
     FT_HIP(hipStreamSynchronize(e->s_h2d));
@@ -171,17 +173,24 @@ int resize_slots(Engine* e, size_t chunk_elems)
         }
         s.used = false;
     }
-    e->chunk = chunk_elems;
     for (Slot& s : e->slots) {
         float** arrays[3] = {&s.p, &s.m, &s.v};
         for (float** a : arrays) {
             const hipError_t err = hipMalloc(reinterpret_cast<void**>(a), chunk_elems * 4);
             if (err != hipSuccess) {
                 (void)hipGetLastError();
-                return fth::fail(FT_ENOMEM, "hipMalloc(%zu) for a larger chunk failed: %s", chunk_elems * 4, hipGetErrorString(err));
+                for (Slot& t : e->slots) {
+                    float** held[3] = {&t.p, &t.m, &t.v};
+                    for (float** h : held) {
+                        if (*h) (void)hipFree(*h);
+                        *h = nullptr;
+                    }
+                }
+                return fth::fail(FT_ENOMEM, "hipMalloc(%zu) for the staging slots failed: %s", chunk_elems * 4, hipGetErrorString(err));
             }
         }
     }
+    e->chunk = chunk_elems;
     return FT_OK;
 }
 
@@ -430,6 +439,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
         const size_t grown = ((n + kMaxChunksPerStep - 1) / kMaxChunksPerStep + mi - 1) / mi * mi;
         if ((rc = resize_slots(e, grown)) != FT_OK) return rc;
     }
+    if ((in_staged || out_staged) && !e->slots.back().v && (rc = resize_slots(e, e->chunk)) != FT_OK) return rc;
     const size_t chunk = e->chunk;
     for (Slot& s : e->slots) {
         if (stage_g && !s.g) FT_HIP(hipMalloc(&s.g, chunk * 4));
