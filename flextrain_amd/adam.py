@@ -129,7 +129,9 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
         ``half_parameter`` the new parameters are also written there in its dtype.
 
         Resident mode (``full_parameter`` on the GPU): the kernel is enqueued on torch's current
-        stream and the call returns at once. Offloaded mode (``full_parameter`` in pinned host
+        stream and the call returns at once. ``half_parameter`` alone may then live in pinned host
+        memory: the kernel writes it there itself, and the host sees it once the stream has passed
+        the kernel. Offloaded mode (``full_parameter`` in pinned host
         memory): the chunk pipeline is enqueued; with ``blocking`` (default in this mode) the call
         returns when the host arrays hold the new values, as the reference's host step does. With
         ``blocking=False`` the call returns at once; torch's current stream is then made to wait
@@ -169,6 +171,8 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             for name, t in (("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq), ("gradient", gradient),
                             ("half_parameter", half_parameter)):
                 if t is not None and t.device != full_parameter.device:
+                    if name == "half_parameter" and not t.is_cuda and t.is_pinned():
+                        continue  # the kernel writes the copy into pinned host memory over the link
                     raise ValueError(f"{name} is on {t.device} but full_parameter is on {full_parameter.device}")
             with torch.cuda.device(full_parameter.device):
                 _C.check("ft_adam_step", self._lib.ft_adam_step(

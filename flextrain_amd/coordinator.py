@@ -22,14 +22,17 @@ What changes because the optimizer runs on the GPU:
     share from there; ordering is by events on the buffers involved, never by a device-wide
     synchronisation (``:819-823``);
   * the updated low-precision parameters are written by the update kernel straight into the
-    unit's parameter buffer in HBM: no H2D copy of new parameters afterwards.
+    unit's parameter buffer in HBM: no H2D copy of new parameters afterwards. A unit whose
+    parameters are kept partly or wholly in pinned host memory (the reference's GPU part + CPU
+    part, ``coordinator/parameter.py:470-519``) gets each element's new value in the piece that
+    holds it, written over the link by the same step.
 Left out (other subsystems): the forward/backward alpha split with borrowed buffers, the NVMe
 tier, gradient reduce-scatter across ranks. Global-norm clipping cannot be combined with
 stepping during backward (the norm is known only after the last unit) and is not offered here.
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import List, Optional, Sequence, Union
 
 import torch
 from torch import Tensor
@@ -61,9 +64,10 @@ class FlexTrainOptsCoordinator:
     def initialize(
         self,
         optimizer: FlexTrainOptimizer,
-        unit_half_parameters: Sequence[Tensor],
+        unit_half_parameters: Sequence[Union[Tensor, Sequence[Tensor]]],
         micro_batch_per_rank: int,
         *,
+        device: Optional[torch.device] = None,
         gradacc_dtype: Optional[torch.dtype] = None,
         offload: bool = True,
         unit_windows: Optional[bool] = None,
@@ -73,8 +77,15 @@ class FlexTrainOptsCoordinator:
         Args:
             optimizer: supplies ``cpu_optimizer`` (the step engine) and ``unit_group_segments``
                 (which parameter group owns which element range of each unit).
-            unit_half_parameters: one flat GPU tensor per unit holding the unit's low-precision
-                parameters, all of the same (padded) length. The update writes new values here.
+            unit_half_parameters: per unit, the flat buffer holding the unit's low-precision
+                parameters, all units of the same (padded) length: one GPU tensor, or a list of
+                pieces that follow one another, each on the GPU or in pinned host memory, cut
+                alike in every unit (the reference keeps a unit's parameters as a GPU part and a
+                CPU part, ``coordinator/parameter.py:470-519``). The update writes the new values
+                into whichever piece holds an element; pieces on the host are written over the
+                link by the step itself and are complete after ``clear_backward_pipeline()``.
+            device: GPU the gradients live on (default: that of the first GPU piece, else the
+                current device).
             micro_batch_per_rank: number of equal shares a unit's step is cut into; the unit
                 length must be divisible by it.
             gradacc_dtype: dtype of the gradient buffers (default: the parameters' dtype).
@@ -90,12 +101,18 @@ class FlexTrainOptsCoordinator:
                 themselves instead of being copied back in one piece after the unit's last share
                 (slower: 43.7 GB/s on the same schedule).
         """
-        units = list(unit_half_parameters)
-        assert units and all(t.is_cuda and t.dim() == 1 and t.is_contiguous() for t in units)
+        units = [[u] if isinstance(u, Tensor) else list(u) for u in unit_half_parameters]
+        assert units and all(units)
+        pieces = [t for u in units for t in u]
+        assert all(t.dim() == 1 and t.is_contiguous() and (t.is_cuda or t.is_pinned()) for t in pieces), \
+            "low-precision parameter pieces must be flat and on the GPU or in pinned host memory"
+        assert all(t.dtype == pieces[0].dtype for t in pieces)
         self._optimizer = optimizer
         self._num_units = len(units)
-        self._unit_numel = units[0].numel()
-        assert all(t.numel() == self._unit_numel for t in units)
+        self._half_piece_numels = [t.numel() for t in units[0]]
+        self._unit_numel = sum(self._half_piece_numels)
+        assert all([t.numel() for t in u] == self._half_piece_numels for u in units), \
+            "every unit must be cut into the same pieces"
         assert self._unit_numel % micro_batch_per_rank == 0
         self._micro_batch_per_rank = micro_batch_per_rank
         self._unit_half_parameters = units
@@ -106,8 +123,11 @@ class FlexTrainOptsCoordinator:
         self._unit_windows = bool(unit_windows) and self._offload
         self._open_windows = {}  # unit index -> window token
         self._window_write_through = bool(window_write_through)
-        device = units[0].device
-        device_dtype = units[0].dtype
+        if device is None:
+            on_gpu = [t.device for t in pieces if t.is_cuda]
+            device = on_gpu[0] if on_gpu else torch.device("cuda", torch.cuda.current_device())
+        device = torch.device(device)
+        device_dtype = pieces[0].dtype
         master_dtype = torch.float32
         self._emit_half = device_dtype != master_dtype
         if not self._emit_half:
@@ -136,10 +156,9 @@ class FlexTrainOptsCoordinator:
             self._unit_numel, (self._num_units, per_element), master_dtype, state_device)
 
         # Seed the master copy from the low-precision parameters (exact: widening conversion).
-        for u, half in enumerate(units):
-            self._unit_opts[u][0].copy_(half)
-        if self._offload:
-            torch.cuda.current_stream(device).synchronize()
+        for u in range(self._num_units):
+            self._copy_master_to_or_from_half(u, to_half=False)
+        torch.cuda.current_stream(device).synchronize()
 
         # One container per unit: equal shares x parameter groups; every buffer is one piece.
         n = [self._unit_numel]
@@ -148,8 +167,20 @@ class FlexTrainOptsCoordinator:
             segments = optimizer.unit_group_segments[u]
             assert segments and segments[-1].end == self._unit_numel, \
                 "unit group segments must cover the padded unit (see FlexTrainOptimizer(aligned_unit_numel=...))"
-            self._unit_step_ctxts.append(StepContextContainer(micro_batch_per_rank, segments, n, n, n))
+            self._unit_step_ctxts.append(StepContextContainer(micro_batch_per_rank, segments, self._half_piece_numels, n, n))
         self._initialized = True
+
+    def _copy_master_to_or_from_half(self, unit_index: int, to_half: bool) -> None:
+        """Piece by piece: seeds the fp32 master copy from the low-precision parameters (exact), or
+        rounds the master copy back into them."""
+        master, offset = self._unit_opts[unit_index][0], 0
+        for piece in self._unit_half_parameters[unit_index]:
+            part = master[offset:offset + piece.numel()]
+            if to_half:
+                piece.copy_(part)
+            else:
+                part.copy_(piece)
+            offset += piece.numel()
 
     # ---- buffers -------------------------------------------------------------------------------
     @property
@@ -279,7 +310,7 @@ class FlexTrainOptsCoordinator:
                                checkpoint_interval=checkpoint_interval)
                 for dst, src in zip(self._unit_opts[u], staging):
                     dst.copy_(src)
-            self._unit_half_parameters[u].copy_(self._unit_opts[u][0])
+            self._copy_master_to_or_from_half(u, to_half=True)
         torch.cuda.current_stream().synchronize()
 
 

@@ -17,8 +17,23 @@ class _Unit:
 
 @pytest.mark.parametrize("offload,windows", [(True, "copy_back"), (True, "write_through"), (True, "off"), (True, "auto"), (False, "off")])
 def test_backward_pipeline_matches_oracle(cuda, oracle, offload, windows):
+    _run_backward_pipeline(cuda, oracle, offload, windows, "gpu")
+
+
+@pytest.mark.parametrize("half_layout", ["split", "split_odd", "host"])
+@pytest.mark.parametrize("offload,windows", [(True, "copy_back"), (True, "off"), (False, "off")])
+def test_half_parameters_on_gpu_and_host_pieces(cuda, oracle, offload, windows, half_layout):
+    """The reference keeps a unit's low-precision parameters as a GPU part and a CPU part
+    (``coordinator/parameter.py:470-519``): the update must write each element's new 16-bit value
+    into the piece that holds it, wherever the cut falls (also at an odd element, where the vector
+    alignments of the arrays disagree), for resident and offloaded master state."""
+    _run_backward_pipeline(cuda, oracle, offload, windows, half_layout)
+
+
+def _run_backward_pipeline(cuda, oracle, offload, windows, half_layout):
     from flextrain_amd import FlexTrainAdam
     from flextrain_amd.coordinator import FlexTrainOptsCoordinator
+    from flextrain_amd.memory import pinned_empty
     torch.manual_seed(0)
     num_units, micro_batches, unit_numel = 4, 4, 1 << 20
     real = unit_numel - 4097  # the tail of each unit is alignment padding
@@ -37,8 +52,26 @@ def test_backward_pipeline_matches_oracle(cuda, oracle, offload, windows):
                         aligned_unit_numel=unit_numel, offload=offload)
     assert opt.non_layerwise_numel == 0
     assert [(s.start, s.end) for s in opt.unit_group_segments[0]] == [(0, w_numel), (w_numel, unit_numel)]
+    # where the coordinator finds (and leaves) the low-precision parameters of each unit
+    cut = {"gpu": unit_numel, "split": 600_064, "split_odd": 600_001, "host": 0}[half_layout]
+    halves = []
+    for u in range(num_units):
+        pieces = []
+        if cut:
+            pieces.append(flat[u] if cut == unit_numel else flat[u][:cut].clone())
+        if cut < unit_numel:
+            host_piece = pinned_empty(unit_numel - cut, torch.bfloat16)
+            host_piece.copy_(flat[u][cut:])
+            pieces.append(host_piece)
+        halves.append(pieces[0] if half_layout == "gpu" else pieces)
+    torch.cuda.synchronize()
+
+    def half_of(u):
+        pieces = [halves[u]] if half_layout == "gpu" else halves[u]
+        return torch.cat([piece.to(cuda) for piece in pieces])
+
     coord = FlexTrainOptsCoordinator()
-    coord.initialize(opt, flat, micro_batches, offload=offload,
+    coord.initialize(opt, halves, micro_batches, offload=offload, device=cuda,
                      unit_windows={"auto": None, "off": False}.get(windows, True),
                      window_write_through=windows == "write_through")
     assert coord._unit_windows == (offload and windows != "off")  # small shares: the automatic choice is windows
@@ -73,12 +106,12 @@ def test_backward_pipeline_matches_oracle(cuda, oracle, offload, windows):
                 pn[lo:hi], mn[lo:hi], vn[lo:hi], hn[lo:hi] = ps, ms, vs, hs
             m, v = coord.unit_optimizer_states(u)
             worst = dict(p=max_ulp(to_np(coord.unit_master_parameter(u)), pn), m=max_ulp(to_np(m), mn),
-                         v=max_ulp(to_np(v), vn), h=max_ulp(half_bits(flat[u]), hn, bf16=True))
-            print(f"[coordinator offload={offload} windows={windows} it={iteration} unit={u}] worst ULP distance: {worst}", flush=True)
+                         v=max_ulp(to_np(v), vn), h=max_ulp(half_bits(half_of(u)), hn, bf16=True))
+            print(f"[coordinator offload={offload} windows={windows} half={half_layout} it={iteration} unit={u}] worst ULP distance: {worst}", flush=True)
             assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst["h"] <= HALF_ULP
     assert decay["step"] == 2 and plain["step"] == 2
-    # the module's parameters are views of the flat unit buffers: they saw the update
-    assert weights[0].data_ptr() == flat[0].data_ptr()
+    if half_layout == "gpu":  # the module's parameters are views of the flat unit buffers: they saw the update
+        assert weights[0].data_ptr() == flat[0].data_ptr() and halves[0] is flat[0]
 
 
 def test_wider_accumulation_type(cuda, oracle):
