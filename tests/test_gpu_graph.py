@@ -1,7 +1,9 @@
 """The resident mixed-precision step (statistics -> decision -> update) allocates nothing and
 clears nothing with memset, so it can be recorded into a HIP graph. The graph is replayed several
 times with eager work and synchronisations in between; every replay is checked against the
-oracle, including one whose gradients overflow (the device-side decision skips it)."""
+oracle, including one whose gradients overflow (the device-side decision skips it). The same for
+the gradient hand-off (fused accumulate / clear / statistics) in front of the step, checked against
+the eager calls."""
 import numpy as np
 import pytest
 import torch
@@ -83,3 +85,89 @@ def test_resident_step_replays_in_a_hip_graph(cuda, oracle):
     # the buffers around the slices were never touched
     for k in "pmv":
         assert not bufs[k][:offset].any() and not bufs[k][offset + n:].any()
+
+
+def test_gradient_hand_off_and_step_replay_in_a_hip_graph(cuda):
+    """Two micro-batches folded into an fp32 accumulator by the fused pass (the second one also
+    gathers the statistics), the device-side decision, and the update consuming the accumulator:
+    recorded once, replayed five times between eager work (one replay with an overflowing
+    micro-batch). Every replay must leave exactly what the same calls leave when run eagerly on
+    copies of the same state."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.loss_scaler import GradientGuard
+    n, scale, t = 2_500_003, 512.0, 7
+    gen = torch.Generator(device=cuda).manual_seed(23)
+
+    def make_state():
+        return dict(p=torch.empty(n, device=cuda), m=torch.empty(n, device=cuda), v=torch.empty(n, device=cuda),
+                    h=torch.zeros(n, dtype=torch.bfloat16, device=cuda), acc=torch.zeros(n, device=cuda),
+                    g=[torch.zeros(n, dtype=torch.float16, device=cuda) for _ in range(2)])
+
+    live, twin = make_state(), make_state()
+    live["p"].copy_(torch.randn(n, device=cuda, generator=gen) * 0.02)
+    live["m"].copy_(torch.randn(n, device=cuda, generator=gen) * 1e-4)
+    live["v"].copy_(torch.rand(n, device=cuda, generator=gen) * 1e-6)
+    eng = FlexTrainCPUAdam(**HP)
+    guards = {id(live): GradientGuard(cuda), id(twin): GradientGuard(cuda)}
+    group = {"step": t}
+
+    def sequence(s):
+        guard = guards[id(s)]
+        guard.begin()
+        guard.accumulate(s["acc"], s["g"][0], scale=0.5, zero_grads=True)
+        guard.accumulate(s["acc"], s["g"][1], scale=0.5, zero_grads=True, with_stats=True, loss_scale=scale)
+        ctl = guard.decide_async(loss_scale=scale, max_grad_norm=1.0)
+        eng._step(group, s["h"], s["p"], s["acc"], s["m"], s["v"], control=ctl)
+
+    def sync_twin():
+        for k in "pmvh":
+            twin[k].copy_(live[k])
+        twin["acc"].copy_(live["acc"])
+        for a, b in zip(twin["g"], live["g"]):
+            a.copy_(b)
+
+    def fresh_gradients(overflow):
+        live["acc"].zero_()
+        for k, g in enumerate(live["g"]):
+            g.copy_((torch.randn(n, device=cuda, generator=gen) * (1e-3 * scale)).to(torch.float16))
+        if overflow:
+            live["g"][1][n - 5] = float("nan")
+
+    # eager warm-up on a side stream (sizes the guard's workspace), undone afterwards, then capture
+    fresh_gradients(False)
+    snapshot = {k: live[k].clone() for k in "pmvh"}
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sequence(live)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        sequence(live)
+    torch.cuda.synchronize()
+    for k in "pmvh":
+        live[k].copy_(snapshot[k])
+
+    for replay, overflow in enumerate([False, True, False, False, False]):
+        fresh_gradients(overflow)
+        sync_twin()
+        torch.cuda.synchronize()
+        graph.replay()
+        sequence(twin)  # the same calls, eagerly, on the copies
+        torch.cuda.synchronize()
+        got, want = guards[id(live)].read(), guards[id(twin)].read()
+        assert got.overflow == want.overflow == overflow
+        assert got.nonfinite == want.nonfinite and got.sumsq == want.sumsq and got.grad_mult == want.grad_mult
+        for k in "pmvh":
+            assert torch.equal(live[k].view(torch.int32 if k != "h" else torch.int16),
+                               twin[k].view(torch.int32 if k != "h" else torch.int16)), f"replay {replay}: {k} differs"
+        assert torch.equal(live["acc"], twin["acc"]) or overflow  # NaN != NaN
+        assert not live["g"][0].any() and not live["g"][1].any()  # sources cleared by the replay
+        if not overflow:
+            assert not torch.equal(live["p"], snapshot["p"])
+            snapshot["p"] = live["p"].clone()
+        print(f"[graph hand-off replay {replay} overflow={overflow}] norm {got.grad_norm:.6g} clip {got.clip_coef:.6g}: equal to eager", flush=True)
+        eager_other = torch.randn(4099, device=cuda)  # unrelated eager work through the same library
+        guards[id(twin)].begin(); guards[id(twin)].add(eager_other)
+        torch.cuda.synchronize()
