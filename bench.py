@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the optimizer-step hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5|pipeline|accumulate] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5|pipeline|accumulate|resident7b] [--no-cpu-baseline]
 
 A "step" is one fused AdamW update over one synthetic partition that is already resident in HBM.
 Default workload: the Llama-7B decoder-layer partition (202,383,360 elements, bf16 gradients,
@@ -390,7 +390,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate", "resident7b"])
     ap.add_argument("--micro-batches", type=int, default=4, help="pipeline: shares per unit")
     ap.add_argument("--windows", default="auto", choices=["auto", "off", "write_through", "copy_back"],
                     help="pipeline: keep a whole unit's state on the GPU while it is stepped (prefetched one unit ahead)")
@@ -429,6 +429,13 @@ def main() -> int:
         n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.bfloat16, 100, 1.0, None
         p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev)
         name = "cfg2: Llama-7B decoder-layer partition resident in HBM, bf16 grads, AdamW t=100, bf16 copy-out"
+        bytes_per_elem, stats_pass = 28, False
+    elif args.workload == "resident7b":
+        # What 288 GB of HBM allow: the whole 7B optimizer of cfg5 (81 GB of fp32 state + 27 GB of bf16
+        # gradients and parameters) resident, stepped by one launch.
+        n, g_dtype, t_step, scale, max_norm = 32 * N_7B_LAYER + 2 * 4096 * 32000, torch.bfloat16, 100, 1.0, None
+        p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev)
+        name = "resident7b: the whole Llama-7B optimizer of cfg5 (6.74e9 elements, 108 GB) resident in HBM, one launch"
         bytes_per_elem, stats_pass = 28, False
     elif args.workload == "cfg3":
         n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.float16, 100, 65536.0, None
@@ -510,7 +517,7 @@ def main() -> int:
         "hbm_frac_of_peak": achieved / HBM_PEAK_GBPS,
         "roofline": {
             "bound": "hbm", "kernel": "adam_tile_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES[args.workload],
+            "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "algorithmic_bytes_per_launch": alg_bytes, "kernel_ms_avg": upd_avg, "kernel_ms_min": min(upd_ms),
             "kernel_ms_p20_80": percentile_mean(upd_ms),
         },
@@ -522,7 +529,7 @@ def main() -> int:
     if not args.no_cpu_baseline:
         del p, g, m, v, h
         torch.cuda.empty_cache()
-        out["cpu_baseline"] = cpu_baseline(n)
+        out["cpu_baseline"] = cpu_baseline(min(n, N_7B_LAYER))
     print(json.dumps(out), flush=True)
     return 0
 
