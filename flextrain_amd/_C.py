@@ -96,5 +96,17 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise ValueError(f"unsupported dtype {dtype}; expected float32, float16 or bfloat16") from None
 
 
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream_ptr(device=None) -> int:
+    """Handle of torch's current stream on ``device`` (default: the current device)."""
+    if _RAW_STREAM is not None:  # the same handle without building a Stream object (2 us -> 0.3 us)
+        if device is None:
+            index = torch.cuda.current_device()
+        else:
+            index = device.index if isinstance(device, torch.device) else torch.device(device).index
+            if index is None:
+                index = torch.cuda.current_device()
+        return _RAW_STREAM(index)
     return torch.cuda.current_stream(device).cuda_stream
