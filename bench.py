@@ -44,15 +44,16 @@ def percentile_mean(samples, lo=0.2, hi=0.8):
 
 def make_inputs(torch, n, g_dtype, g_std, device, scale=1.0):
     """p, g, m, v and the 16-bit copy of one partition, in the library's own layout for the arrays
-    of an update (one allocation, staggered starts), filled in place from a seeded generator."""
+    of an update (one allocation, staggered starts), filled in place by the seeded generator
+    (seed 0, one substream per array: the same values on any machine, on the GPU and on the host)."""
+    from flextrain_amd import synth
     from flextrain_amd.memory import allocate_device_arrays
-    gen = torch.Generator(device=device).manual_seed(0)
     p, m, v, g, h = allocate_device_arrays(
         [(n, torch.float32)] * 3 + [(n, g_dtype), (n, torch.bfloat16)], device)
-    p.normal_(0.0, 0.02, generator=gen)
-    m.normal_(0.0, 1e-4, generator=gen)
-    v.uniform_(0.0, 1e-6, generator=gen)
-    g.normal_(0.0, g_std * scale, generator=gen)
+    synth.fill_(p, 0, 0, scale=0.02)
+    synth.fill_(m, 0, 1, scale=1e-4)
+    synth.fill_(v, 0, 2, kind=synth.UNIFORM, scale=1e-6)
+    synth.fill_(g, 0, 3, scale=g_std * scale)
     return p, g, m, v, h
 
 
@@ -248,8 +249,9 @@ def bench_accumulate(args, torch, dev) -> int:
     n = N_7B_LAYER
     guard = GradientGuard(dev)
     from flextrain_amd.memory import allocate_device_arrays
+    from flextrain_amd import synth
     acc, g = allocate_device_arrays([(n, torch.float32), (n, torch.bfloat16)], dev)
-    g.normal_(0.0, 1e-3, generator=torch.Generator(device=dev).manual_seed(0))
+    synth.fill_(g, 0, 3, scale=1e-3)
     if args.calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
         scratch = torch.empty_like(acc)
         for _ in range(3):
@@ -391,19 +393,19 @@ def bench_resident7b(args, torch, dev) -> int:
     lm_head), as the coordinator lays resident state out, and one launch per unit: the arrays of a
     launch then lie within a few GB of each other, which the kernel rewards (the same kernel over
     five 27 GB arrays in one launch runs at 82.6 % of peak instead of 85 %)."""
-    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd import FlexTrainCPUAdam, synth
     from flextrain_amd.memory import allocate_device_arrays
     eng = FlexTrainCPUAdam(**HP)
     sizes = [N_7B_LAYER] * 32 + [2 * 4096 * 32000]
-    gen = torch.Generator(device=dev).manual_seed(0)
-    units = []
-    for n in sizes:
+    units, first = [], 0
+    for n in sizes:  # the units are consecutive element ranges of the four substreams
         p, m, v, g, h = allocate_device_arrays([(n, torch.float32)] * 3 + [(n, torch.bfloat16)] * 2, dev)
-        p.normal_(0.0, 0.02, generator=gen)
-        m.normal_(0.0, 1e-4, generator=gen)
-        v.uniform_(0.0, 1e-6, generator=gen)
-        g.normal_(0.0, 1e-3, generator=gen)
+        synth.fill_(p, 0, 0, scale=0.02, first_index=first)
+        synth.fill_(m, 0, 1, scale=1e-4, first_index=first)
+        synth.fill_(v, 0, 2, kind=synth.UNIFORM, scale=1e-6, first_index=first)
+        synth.fill_(g, 0, 3, scale=1e-3, first_index=first)
         units.append((h, p, g, m, v))
+        first += n
     total = sum(sizes)
     group = {"step": 100}
 

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_uint64, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_size_t, c_uint32, c_uint64, c_void_p
 
 import torch
 
@@ -47,6 +47,8 @@ EXPORTS = {
     "ft_offload_wait": (c_int, [c_void_p]),
     "ft_offload_elapsed_ms": (c_int, [c_void_p, POINTER(c_float)]),
     "ft_link_bandwidth": (c_int, [c_size_t, c_int, c_int, POINTER(c_double)]),
+    "ft_synth_fill": (c_int, [c_void_p, c_int, c_size_t, c_uint64, c_uint32, c_uint64, c_int, c_float, c_void_p]),
+    "ft_synth_fill_host": (c_int, [c_void_p, c_int, c_size_t, c_uint64, c_uint32, c_uint64, c_int, c_float]),
     "ft_set_launch_tuning": (c_int, [c_int, c_int]),
 }
 

@@ -15,7 +15,7 @@ _ROOT = os.path.dirname(_PKG)
 CSRC = os.path.join(_PKG, "csrc")
 INCLUDE = os.path.join(_ROOT, "include")
 LIB_PATH = os.path.join(_PKG, "libftadam.so")
-SOURCES = ("ft_adam.hip", "ft_offload.hip")
+SOURCES = ("ft_adam.hip", "ft_offload.hip", "ft_synth.hip")
 
 # -ffp-contract=off: the kernels spell out every fused multiply-add; the compiler must not form
 #   others, or results would differ from the reference's operation sequence.

@@ -199,6 +199,24 @@ int ft_offload_elapsed_ms(void* handle, float* out_ms);
  * The method follows the reference's own probe (flextrain/auto_config.py:184-215). */
 int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps);
 
+/* ---- synthetic inputs ----------------------------------------------------------------------
+ * Seeded benchmark / test inputs whose element i is a pure function of (seed, substream,
+ * first_index + i): 64-bit counter hash -> 24-bit uniforms -> (FT_SYNTH_NORMAL) Box-Muller with the
+ * logarithm, cosine and 16-bit conversions written out in IEEE fp32 / integer operations, so the
+ * device fill and the host fill give the same bits on any machine and for any chunking of a large
+ * array. The reference draws its probe inputs with torch.randn on the host
+ * (flextrain/optimizer.py:71-95 via flextrain/auto_config.py:281-317), which cannot be reproduced
+ * elsewhere without shipping the data.
+ * FT_SYNTH_NORMAL: mean 0, standard deviation `scale`; FT_SYNTH_UNIFORM: (0, scale].
+ * ft_synth_fill writes device (or pinned host) memory from a kernel on `stream`;
+ * ft_synth_fill_host writes host memory from the calling thread and needs no GPU. */
+#define FT_SYNTH_NORMAL 0
+#define FT_SYNTH_UNIFORM 1
+int ft_synth_fill(void* out, int dtype, size_t n, uint64_t seed, uint32_t substream, uint64_t first_index,
+                  int kind, float scale, void* stream);
+int ft_synth_fill_host(void* out, int dtype, size_t n, uint64_t seed, uint32_t substream, uint64_t first_index,
+                       int kind, float scale);
+
 /* ---- launch tuning ------------------------------------------------------------------------
  * adam_waves_per_cu: how many 64-lane workgroups of the update kernel (16-bit gradients: 56 bytes
  * of loads in flight per lane) may be resident on one compute unit; kernels with fewer bytes per

@@ -230,6 +230,30 @@ void offloaded_step(hipStream_t stream)
     HIP_OK(hipFree(dg)); HIP_OK(hipFree(dh));
 }
 
+// The seeded input generator: the kernel and the host loop must give the same bits.
+void synthetic_inputs(hipStream_t stream)
+{
+    const size_t n = 100003;
+    const uint64_t first = (1ull << 33) + 5;
+    for (int dtype : {FT_F32, FT_F16, FT_BF16}) {
+        const size_t esz = dtype == FT_F32 ? 4 : 2;
+        std::vector<unsigned char> host(n * esz), back(n * esz);
+        void* dev = nullptr;
+        HIP_OK(hipMalloc(&dev, n * esz));
+        for (int kind : {FT_SYNTH_NORMAL, FT_SYNTH_UNIFORM}) {
+            FT_OK_OR_DIE(ft_synth_fill(dev, dtype, n, 0, 3, first, kind, 1e-3f, stream));
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipMemcpy(back.data(), dev, n * esz, hipMemcpyDeviceToHost));
+            FT_OK_OR_DIE(ft_synth_fill_host(host.data(), dtype, n, 0, 3, first, kind, 1e-3f));
+            char what[96];
+            std::snprintf(what, sizeof what, "synthetic inputs, dtype %d kind %d: device fill == host fill", dtype, kind);
+            check(!std::memcmp(host.data(), back.data(), n * esz), what);
+        }
+        HIP_OK(hipFree(dev));
+    }
+    check(ft_synth_fill(nullptr, FT_F32, 4, 0, 0, 0, FT_SYNTH_NORMAL, 1.f, stream) == FT_EINVAL, "synthetic fill rejects a NULL target");
+}
+
 }  // namespace
 
 int main()
@@ -245,6 +269,7 @@ int main()
     resident_mixed_precision_step(stream);
     accumulate_pass(stream);
     offloaded_step(stream);
+    synthetic_inputs(stream);
     HIP_OK(hipStreamDestroy(stream));
     std::printf("%s (%d failed)\n", g_failures ? "FAILED" : "ALL PASSED", g_failures);
     return g_failures ? 1 : 0;
