@@ -28,7 +28,7 @@ N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 8
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
 # profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_657_000, "cfg3": 5_666_695_000, "cfg4": 23_958_237_000, "accumulate": 2_453_897_000}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_657_000, "cfg3": 5_666_664_000, "cfg4": 23_958_221_000, "accumulate": 2_453_887_000}
 
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
 
