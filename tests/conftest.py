@@ -12,6 +12,17 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+@pytest.fixture(scope="session", autouse=True)
+def built_library():
+    """The tests load the library that is built in-tree; only a tree where nothing has been built
+    yet (a fresh clone) compiles it first."""
+    from flextrain_amd import _C
+    if not os.path.exists(_C.LIB_PATH):
+        from flextrain_amd.build import build_library
+        build_library()
+    return _C.LIB_PATH
+
+
 @pytest.fixture(scope="session")
 def oracle():
     """The CPU checker (test infrastructure)."""
