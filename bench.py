@@ -530,8 +530,11 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
-    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd import FlexTrainCPUAdam, _C
     from flextrain_amd.loss_scaler import GradientGuard
+    if not os.path.exists(_C.LIB_PATH):  # nothing built in this tree yet
+        from flextrain_amd.build import build_library
+        build_library()
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
