@@ -210,6 +210,53 @@ def test_every_operation_rounds_once_in_the_reference_order(oracle, adamw_mode, 
         assert (F(p[i]), F(m[i]), F(v[i])) == want[i], i
 
 
+def exact_trace(s, p, g, m, v, grad_mult=1.0):
+    """All eleven intermediates of exact_step, in the order of oracle.TRACE_NAMES."""
+    g = fl32(F(g) * F(grad_mult))
+    if s.wd_mode == 2:
+        g = fl32(F(p) * F(s.wd_coef) + g)
+    m1 = fl32(F(m) * F(s.beta1))
+    mn = fl32(g * F(s.omb1) + m1)
+    v1 = fl32(F(v) * F(s.beta2))
+    g2 = fl32(g * g)
+    vn = fl32(g2 * F(s.omb2) + v1)
+    sq = fl32_sqrt(vn)
+    d = fl32(sq * F(s.bias2) + F(s.eps))
+    u = fl32(mn / d)
+    p1 = fl32(F(p) * F(s.wd_coef) + F(p)) if s.wd_mode == 1 else F(p)
+    pn = fl32(u * F(s.step_size) + p1)
+    return dict(zip(("g32", "m1", "m_new", "v1", "g2", "v_new", "sqrt", "denom", "update", "p1", "p_new"),
+                    (g, m1, mn, v1, g2, vn, sq, d, u, p1, pn)))
+
+
+@pytest.mark.parametrize("adamw_mode,wd", [(True, 0.01), (True, 0.0), (False, 0.01)])
+def test_trace_exposes_the_same_intermediates(oracle, adamw_mode, wd):
+    """adam_trace (one element, every intermediate) against exact rationals rounded once per
+    operation, for the three weight-decay modes; its p', m', v' are those of adam_step. A trace
+    that skipped the L2 term, decayed after the update or reported a value from the wrong line
+    would differ in some named entry."""
+    rng = np.random.default_rng(21)
+    n = 200
+    p = rng.normal(0, 0.02, n).astype(np.float32)
+    g = rng.normal(0, 1e-3, n).astype(np.float32)
+    m = rng.normal(0, 1e-4, n).astype(np.float32)
+    v = rng.uniform(0, 1e-6, n).astype(np.float32)
+    mult = float(np.float32(0.61))
+    s = oracle.scalars(step=7, lr=2e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=wd, adamw_mode=adamw_mode)
+    assert s.wd_mode == (0 if wd == 0.0 else (1 if adamw_mode else 2))
+    traces = [oracle.adam_trace(s, float(p[i]), float(g[i]), float(m[i]), float(v[i]), grad_mult=mult) for i in range(n)]
+    for i in range(n):
+        want = exact_trace(s, p[i], g[i], m[i], v[i], mult)
+        assert set(traces[i]) == set(want)
+        for name, value in want.items():
+            assert F(traces[i][name]) == value, (i, name)
+    ps, ms, vs = p.copy(), m.copy(), v.copy()
+    oracle.adam_step(ps, g, ms, vs, step=7, lr=2e-4, weight_decay=wd, adamw_mode=adamw_mode, grad_mult=mult)
+    assert np.array_equal(ps, np.array([t["p_new"] for t in traces], np.float32))
+    assert np.array_equal(ms, np.array([t["m_new"] for t in traces], np.float32))
+    assert np.array_equal(vs, np.array([t["v_new"] for t in traces], np.float32))
+
+
 def test_host_scalars_follow_the_reference_types(oracle):
     """beta^t in double then float; everything after in float (cpu_adam.h:67-102,148-166)."""
     for t in (1, 2, 10, 100, 1000, 12345):
@@ -434,6 +481,15 @@ def test_clip_coefficient_and_multiplier(oracle):
     norm = torch.nn.utils.clip_grad_norm_([t], max_norm=1.0)
     assert torch.allclose(t.grad, g0 * oracle.clip_coefficient(float(norm), 1.0), rtol=1e-6)
     assert oracle.combined_multiplier(65536.0, 1.0) == np.float32(2.0 ** -16)
+    # Scales that are no power of two with a clip below 1: the multiplier is the fp32 product of the
+    # two separately rounded factors, fl(fl(clip) * fl(1/scale)). The cases are chosen (and checked)
+    # so that the other plausible readings -- fl(clip/scale), or the product formed in double and
+    # rounded once -- give a different float.
+    for scale, clip in ((3.0, 0.839667), (65535.0, 0.543673), (1000.0, 0.014088), (48000.0, 0.915513), (100.0, 0.301756)):
+        a, b = fl32(Fraction(clip)), fl32(Fraction(1.0 / scale))
+        want = fl32(a * b)
+        assert fl32(Fraction(clip) / Fraction(scale)) != want and fl32(Fraction(clip) * Fraction(1.0 / scale)) != want
+        assert F(oracle.combined_multiplier(scale, clip)) == want, (scale, clip)
 
 
 def test_loss_scale_traces(oracle):
