@@ -158,20 +158,32 @@ __device__ __forceinline__ f32x4 load_g4(const void* g, uint64_t unit)
 // is no bounds check and no loop.
 // Inputs and outputs are the same arrays for an in-place update; the offloaded step may point the
 // outputs elsewhere (staging buffer -> host memory, or the reverse), hence no __restrict__.
-// HT == -1: no low-precision copy. HAS_CTL: a.ctl is read first; a skipped step touches nothing
-// else (measured: looking at the decision before or after issuing the vector loads makes no
+// HT == -1: no low-precision copy. HAS_CTL: a.ctl is read first; a skipped in-place step touches
+// nothing else (measured: looking at the decision before or after issuing the vector loads makes no
 // difference to a normal step, 0.835 against 0.833 ms; a skipped step costs 0.17 ms of workgroup
-// dispatch the first way and 0.40 ms the second).
+// dispatch the first way and 0.40 ms the second). The low-precision copy is never written on a
+// skip: it has no input to copy from, so a caller that skips must not stage it.
 template <int GT, int HT, bool HAS_CTL>
 __global__ __launch_bounds__(kWave) void adam_tile_kernel(AdamArgs a, uint64_t tile0)
 {
     AdamConsts c = a.c;
-    if constexpr (HAS_CTL) {  // wave-uniform scalar loads: one decision per step
-        if (a.ctl->skip) return;
-        c.grad_mult = a.ctl->grad_mult;
-    }
     const uint64_t t0 = (tile0 + blockIdx.x) * kWave;  // first unit of the tile: wave-uniform
     const uint64_t i = t0 + threadIdx.x;
+    if constexpr (HAS_CTL) {  // wave-uniform scalar loads: one decision per step
+        if (a.ctl->skip) {
+            // A skipped step leaves the state as it is. Where the outputs are other arrays than
+            // the inputs (a staging buffer on one side of the host link) "as it is" still has to
+            // arrive there: whatever is copied onwards from the outputs must be the old state.
+            if (a.p_out != a.p) st_stream(tile_rsrc(reinterpret_cast<f32x4*>(a.p_out) + t0, kWave * 16), threadIdx.x * 16,
+                                          ld<true>(reinterpret_cast<const f32x4*>(a.p) + i));
+            if (a.m_out != a.m) st_stream(tile_rsrc(reinterpret_cast<f32x4*>(a.m_out) + t0, kWave * 16), threadIdx.x * 16,
+                                          ld<true>(reinterpret_cast<const f32x4*>(a.m) + i));
+            if (a.v_out != a.v) st_stream(tile_rsrc(reinterpret_cast<f32x4*>(a.v_out) + t0, kWave * 16), threadIdx.x * 16,
+                                          ld<true>(reinterpret_cast<const f32x4*>(a.v) + i));
+            return;
+        }
+        c.grad_mult = a.ctl->grad_mult;
+    }
     f32x4 g = load_g4<GT, true>(a.g, i);
     f32x4 p = ld<true>(reinterpret_cast<const f32x4*>(a.p) + i);
     f32x4 m = ld<true>(reinterpret_cast<const f32x4*>(a.m) + i);
@@ -198,11 +210,19 @@ template <int GT, int HT>
 __global__ __launch_bounds__(256) void adam_scalar_kernel(AdamArgs a)
 {
     AdamConsts c = a.c;
+    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
     if (a.ctl) {
-        if (a.ctl->skip) return;
+        if (a.ctl->skip) {  // out of place: the old state still has to reach the outputs
+            if (a.p_out != a.p || a.m_out != a.m || a.v_out != a.v)
+                for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += stride) {
+                    a.p_out[i] = a.p[i];
+                    a.m_out[i] = a.m[i];
+                    a.v_out[i] = a.v[i];
+                }
+            return;
+        }
         c.grad_mult = a.ctl->grad_mult;
     }
-    const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n; i += stride) {
         float g;
         if constexpr (GT == FT_F32)

@@ -433,7 +433,12 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     char* hb = static_cast<char*>(half_out);
 
     const bool stage_g = g_on_host && in_staged;
-    const bool stage_h = half_out && half_on_host && out_staged;
+    // With a control record the step may turn out to be a no-op, and a skipped kernel writes no
+    // low-precision copy: a staged copy-back would then carry whatever the slot held before. The
+    // kernel therefore writes a host-resident copy itself, over the link, and on a skip the host
+    // array keeps its contents. (p, m and v need no such care: a skipped kernel whose outputs are
+    // not its inputs copies the old state through.)
+    const bool stage_h = half_out && half_on_host && out_staged && !ctl;
     if ((in_staged || out_staged) && (n + e->chunk - 1) / e->chunk > kMaxChunksPerStep) {
         const size_t mi = 1u << 20;
         const size_t grown = ((n + kMaxChunksPerStep - 1) / kMaxChunksPerStep + mi - 1) / mi * mi;

@@ -324,6 +324,89 @@ def test_write_through_window(cuda, oracle):
     _assert_equal_bits("write-through window", p, m, v, h, want, torch.bfloat16)
 
 
+def _control(cuda, skip, grad_mult):
+    """A device ft_step_control_t: {u32 skip, f32 grad_mult, f32 grad_norm, f32 clip_coef}."""
+    ctl = torch.zeros(4, dtype=torch.float32, device=cuda)
+    ctl[1], ctl[3] = grad_mult, 1.0
+    ctl.view(torch.int32)[0] = int(skip)
+    return ctl
+
+
+@pytest.mark.parametrize("half_on_host", [True, False])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+def test_device_side_skip_and_multiplier_in_every_transfer_mode(cuda, oracle, mode, half_on_host):
+    """A control record on an offloaded step. Skipped: the host master state and the low-precision
+    copy (in pinned host memory or on the GPU) keep their bits, although the engine's staging slots
+    hold another unit's data from the step before (the poison). Not skipped: the record's
+    multiplier replaces grad_mult and the result equals the oracle's."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.memory import pinned_empty
+    n = 900_001
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 17, offload_slots=2, offload_mode=mode, **HP)
+
+    def half_buffer():
+        if half_on_host:
+            t = pinned_empty(n, torch.float16)
+            t.fill_(3.0)
+            return t
+        return torch.full((n,), 3.0, dtype=torch.float16, device=cuda)
+
+    # poison: a step on other memory leaves its values in the slots (p, m, v and the copy)
+    pp, pm, pv = _host_state(n, seed=90)
+    pp.fill_(777.0)
+    ph = half_buffer()
+    eng._step({"step": 1}, ph, pp, torch.zeros(n, dtype=torch.float16, device=cuda), pm, pv)
+
+    p, m, v = _host_state(n, seed=91)
+    g = (torch.randn(n, device=cuda) * 1e-3 * 1024).to(torch.float16)
+    h = half_buffer()
+    before = tuple(t.clone() for t in (p, m, v))
+    eng._step({"step": 7}, h, p, g, m, v, control=_control(cuda, 1, 1.0 / 1024))
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip((p, m, v), before)), "a skipped step changed the master state"
+    assert bool((h == 3.0).all()), "a skipped step changed the low-precision copy"
+
+    want = _oracle(oracle, p, g, m, v, 7, torch.float16, grad_mult=1.0 / 1024)
+    eng._step({"step": 7}, h, p, g, m, v, grad_mult=55.0, control=_control(cuda, 0, 1.0 / 1024))
+    torch.cuda.synchronize()
+    _assert_equal_bits(f"control mode={mode} half_on_host={half_on_host}", p, m, v, h, want, torch.float16)
+
+
+@pytest.mark.parametrize("write_through", [False, True])
+def test_device_side_skip_inside_a_window(cuda, oracle, write_through):
+    """Shares of a unit stepped inside a window under a control record: a skipped iteration leaves
+    host state and copy alone after the close (copy-back and write-through windows), the next one
+    steps normally."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.memory import pinned_empty
+    n, shares = 800_000, 4
+    per = n // shares
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 16, **HP)
+    warm = _host_state(n, seed=95)  # the window's device arrays hold this unit's values afterwards
+    token = eng.open_window(*warm)
+    eng.close_window(token)
+    p, m, v = _host_state(n, seed=96)
+    before = tuple(t.clone() for t in (p, m, v))
+    g = (torch.randn(n, device=cuda) * 1e-3 * 256).to(torch.float16)
+    h = pinned_empty(n, torch.bfloat16)
+    h.fill_(5.0)
+    for skip in (1, 0):
+        ctl = _control(cuda, skip, 1.0 / 256)
+        want = _oracle(oracle, p, g, m, v, 3, torch.bfloat16, grad_mult=1.0 / 256)
+        token = eng.open_window(p, m, v, write_through=write_through)
+        for k in range(shares):
+            sl = slice(k * per, (k + 1) * per)
+            eng._step({"step": 3}, h[sl], p[sl], g[sl], m[sl], v[sl], control=ctl, blocking=False)
+        eng.close_window(token)
+        eng.synchronize()
+        torch.cuda.synchronize()
+        if skip:
+            assert all(torch.equal(a, b) for a, b in zip((p, m, v), before))
+            assert bool((h == 5.0).all())
+        else:
+            _assert_equal_bits(f"window control write_through={write_through}", p, m, v, h, want, torch.bfloat16)
+
+
 @pytest.mark.parametrize("mode", [1, 3, 4])
 def test_engine_grows_its_chunk_for_long_steps(cuda, oracle, mode):
     """A step that would need more than 96 chunks makes the engine enlarge its chunk first (long
