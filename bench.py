@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the optimizer-step hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5|pipeline|accumulate|resident7b] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5|pipeline|accumulate|resident7b|multi] [--no-cpu-baseline]
 
 A "step" is one fused AdamW update over one synthetic partition that is already resident in HBM.
 Default workload: the Llama-7B decoder-layer partition (202,383,360 elements, bf16 gradients,
@@ -444,6 +444,67 @@ def bench_pipeline_resident(args, torch, dev, Unit) -> int:
     return 0
 
 
+def bench_multi(args, torch, dev) -> int:
+    """The 7B-layer partition of cfg2 cut into --segments ragged contexts of two parameter groups
+    (different weight decay and step count), the way a unit's share reaches the step engine when
+    groups and buffer pieces cut it (flextrain/param_group.py:365-477): all contexts in one launch
+    (ft_adam_step_multi) against one call per context (the reference's loop, flextrain/optimizer.py:44-69)."""
+    import random
+
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.param_group import StepContext
+    n, k = N_7B_LAYER, max(1, args.segments)
+    eng = FlexTrainCPUAdam(**HP)
+    p, g, m, v, h = make_inputs(torch, n, torch.bfloat16, 1e-3, dev)
+    rng = random.Random(0)
+    cuts = sorted({0, n} | {rng.randrange(1, n) for _ in range(k - 1)})
+    groups = [dict(HP, step=100), dict(HP, step=37, weight_decay=0.0)]
+    ctxs = [StepContext(groups[i % 2], h[lo:hi], p[lo:hi], g[lo:hi], [m[lo:hi], v[lo:hi]])
+            for i, (lo, hi) in enumerate(zip(cuts[:-1], cuts[1:]))]
+
+    def one_launch():
+        eng._step_many(ctxs)
+
+    def per_context():
+        for c in ctxs:
+            eng._step(c.param_group, c.half_parameter, c.full_parameter, c.gradient, *c.optimizer_states)
+
+    results = {}
+    for name, fn in (("one_launch", one_launch), ("per_context", per_context)):
+        for _ in range(args.warmup):
+            fn()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        host = 0.0
+        for a, b in ev:
+            a.record()
+            h0 = time.perf_counter()
+            fn()
+            host += time.perf_counter() - h0
+            b.record()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
+        results[name] = {"ms_avg": ms, "achieved_gbps": n * 28 / (ms * 1e-3) / 1e9, "frac": n * 28 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                         "wall_ms_per_step": wall * 1e3 / args.steps, "host_us_per_step": host * 1e6 / args.steps}
+    main = results["one_launch"]
+    print(json.dumps({
+        "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
+        "value": n / (main["wall_ms_per_step"] * 1e-3), "unit": "elements/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": main["wall_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"multi: the cfg2 partition cut into {len(ctxs)} ragged contexts of two parameter groups, "
+                               "stepped by one launch (against one call per context)", "elements": n, "segments": len(ctxs),
+                   "shortest": min(c.full_parameter.numel() for c in ctxs), "longest": max(c.full_parameter.numel() for c in ctxs)},
+        "roofline": {"bound": "hbm", "kernel": "adam_multi_kernel", "achieved": main["achieved_gbps"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": main["frac"], "traffic": None, "algorithmic_bytes_per_launch": n * 28,
+                     "kernel_ms_avg": main["ms_avg"]},
+        "variants": results,
+    }), flush=True)
+    return 0
+
+
 def bench_resident7b(args, torch, dev) -> int:
     """What 288 GB of HBM allow: the whole 7B optimizer of cfg5 (81 GB of fp32 state + 27 GB of bf16
     gradients and parameters) resident. One allocation per unit (32 decoder layers + embedding and
@@ -506,7 +567,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate", "resident7b"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate", "resident7b", "multi"])
+    ap.add_argument("--segments", type=int, default=16, help="multi: ragged contexts the partition is cut into")
     ap.add_argument("--micro-batches", type=int, default=4, help="pipeline: shares per unit")
     ap.add_argument("--windows", default="auto", choices=["auto", "off", "write_through", "copy_back"],
                     help="pipeline: keep a whole unit's state on the GPU while it is stepped (prefetched one unit ahead)")
@@ -546,6 +608,8 @@ def main() -> int:
         return bench_accumulate(args, torch, dev)
     if args.workload == "resident7b":
         return bench_resident7b(args, torch, dev)
+    if args.workload == "multi":
+        return bench_multi(args, torch, dev)
     eng = FlexTrainCPUAdam(**HP)
 
     if args.workload == "cfg2":

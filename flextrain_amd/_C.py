@@ -17,6 +17,17 @@ DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libftadam.so")
 
+class AdamSegment(ctypes.Structure):
+    """Mirror of ``ft_adam_segment_t``: one contiguous piece of an in-place update."""
+
+    _fields_ = [
+        ("p", c_void_p), ("g", c_void_p), ("m", c_void_p), ("v", c_void_p), ("half_out", c_void_p),
+        ("n", c_size_t), ("step", c_uint64),
+        ("lr", c_float), ("beta1", c_float), ("beta2", c_float), ("eps", c_float), ("weight_decay", c_float),
+        ("bias_correction", ctypes.c_int32), ("grad_mult", c_float), ("reserved", ctypes.c_int32),
+    ]
+
+
 EXPORTS = {
     # name: (restype, argtypes)
     "ft_last_error": (c_char_p, []),
@@ -27,6 +38,7 @@ EXPORTS = {
     "ft_adam_step": (c_int, [c_int, c_uint64, c_float, c_float, c_float, c_float, c_float, c_int, c_float,
                              c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_size_t,
                              c_void_p, c_void_p]),
+    "ft_adam_step_multi": (c_int, [c_int, POINTER(AdamSegment), c_int, c_int, c_int, c_void_p, c_void_p]),
     "ft_grad_stats_workspace_bytes": (c_size_t, []),
     "ft_grad_stats": (c_int, [c_void_p, c_int, c_size_t, c_float, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "ft_grad_accumulate_workspace_bytes": (c_size_t, [c_size_t]),

@@ -201,6 +201,58 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             # later work on the caller's stream may overwrite the gradients or read the new copy
             _C.check("ft_offload_stream_wait", self._lib.ft_offload_stream_wait(engine, _C.current_stream_ptr(), 0))
 
+    def _step_many(self, step_contexts, grad_mult: float = 1.0, control: Optional[Tensor] = None) -> None:
+        """Steps resident contexts -- each what one ``_step`` call would take, with its own group
+        hyper-parameters and step count -- in as few kernel launches as possible: up to 16 contexts
+        per launch (``ft_adam_step_multi``), instead of up to three launches per context. The
+        reference loops over the contexts and calls the native step once for each
+        (``flextrain/optimizer.py:44-69``). Results are those of ``_step`` context by context, bit
+        for bit. All contexts must be on one GPU with one gradient dtype; the contexts of a call must
+        not overlap."""
+        live = [ctx for ctx in step_contexts if ctx.gradient.numel()]
+        if not live:
+            return
+        first = live[0]
+        device, g_dtype = first.full_parameter.device, first.gradient.dtype
+        half_dtype = next((c.half_parameter.dtype for c in live if c.half_parameter is not None), torch.float16)
+        ctl_ptr = None
+        if control is not None:
+            if not control.is_cuda or control.numel() * control.element_size() < 16:
+                raise ValueError("control must be a 16-byte device buffer (ft_step_control_t)")
+            ctl_ptr = control.data_ptr()
+        segs = (_C.AdamSegment * len(live))()
+        f32 = {torch.float32}
+        for seg, ctx in zip(segs, live):
+            group = ctx.param_group
+            assert STEP_KEY in group, f"Key '{STEP_KEY}' not found in parameter group arguments."
+            self._set_defaults_args(group)
+            if len(ctx.optimizer_states) != 2:
+                raise ValueError("Adam needs exactly two optimizer states (exp_avg, exp_avg_sq)")
+            full, grad, half = ctx.full_parameter, ctx.gradient, ctx.half_parameter
+            exp_avg, exp_avg_sq = ctx.optimizer_states
+            n = full.numel()
+            _flat("full_parameter", full, f32, n)
+            _flat("exp_avg", exp_avg, f32, n)
+            _flat("exp_avg_sq", exp_avg_sq, f32, n)
+            _flat("gradient", grad, {g_dtype}, n)
+            for name, t in (("full_parameter", full), ("exp_avg", exp_avg), ("exp_avg_sq", exp_avg_sq), ("gradient", grad)):
+                if t.device != device:
+                    raise ValueError(f"{name} is on {t.device}, expected {device}: one call steps one GPU's contexts")
+            if half is not None:
+                _flat("half_parameter", half, {half_dtype}, n)
+                if half.device != device and not (not half.is_cuda and half.is_pinned()):
+                    raise ValueError(f"half_parameter is on {half.device}; it must be on {device} or in pinned host memory")
+                seg.half_out = half.data_ptr()
+            seg.p, seg.g, seg.m, seg.v, seg.n = full.data_ptr(), grad.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), n
+            seg.step, seg.lr = int(group[STEP_KEY]), float(group["lr"])
+            seg.beta1, seg.beta2 = group["betas"]
+            seg.eps, seg.weight_decay = float(group["eps"]), float(group["weight_decay"])
+            seg.bias_correction, seg.grad_mult = int(bool(group["bias_correction"])), float(grad_mult)
+        with torch.cuda.device(device):
+            _C.check("ft_adam_step_multi", self._lib.ft_adam_step_multi(
+                self.opt_id, segs, len(live), _C.dtype_code(g_dtype), _C.dtype_code(half_dtype), ctl_ptr,
+                _C.current_stream_ptr(device)))
+
     def open_window(self, full_parameter: Tensor, exp_avg: Tensor, exp_avg_sq: Tensor, write_through: bool = False) -> int:
         """Brings the whole master state of one unit (three pinned host tensors of equal length) to
         the GPU with large copies and keeps it there until ``close_window``: every ``_step`` on

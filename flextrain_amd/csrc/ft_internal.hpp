@@ -40,6 +40,13 @@ int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, 
                 void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream,
                 float* p_out = nullptr, float* m_out = nullptr, float* v_out = nullptr);
 
+// Elements of a segment that go in front of its vector body (see the definition).
+size_t segment_head(const void* p, size_t n);
+
+// One launch of the many-segment update kernel over the table in `a` (see ft_types.hpp).
+int launch_adam_multi(const ftk::AdamMultiArgs& a, int g_dtype, bool with_half, int half_dtype, unsigned workgroups,
+                      hipStream_t stream);
+
 int cu_count();  // compute units of the current device (cached)
 
 // Dynamic LDS per 64-lane workgroup that keeps the bytes in flight per CU at the tuned level for a

@@ -239,6 +239,105 @@ __global__ __launch_bounds__(256) void adam_scalar_kernel(AdamArgs a)
     }
 }
 
+// Many segments, one launch: the per-(unit, micro-batch) loop of the reference steps one StepContext
+// after the other (flextrain/optimizer.py:44-69), dozens of short calls per unit; here up to
+// kMultiMaxSegments of them, each with its own pointers, length and hyper-parameters, are one grid.
+// Workgroup w belongs to the segment s whose first workgroup is the last one not after w (a scalar
+// compare chain over the table in the kernel-argument segment, then one scalar load of the
+// segment's record from there: no table in device memory). Inside a segment, workgroup
+// k < body_tiles is a full 256-element tile behind the segment's head and runs the straight-line
+// code of adam_tile_kernel; the one workgroup after them takes the segment's edge elements (the
+// head in front of the first tile, up to 255 elements behind the last whole tile) one element per
+// lane and round, through the same adam_element. In place only.
+typedef const char __attribute__((address_space(4))) * KernargBytes;
+
+template <int GT, int HT, bool HAS_CTL>
+__global__ __launch_bounds__(kWave) void adam_multi_kernel(AdamMultiArgs a)
+{
+    // Table entry k = (first workgroup of segment k) << 4 | k, ascending, unused entries all ones:
+    // the largest entry that does not exceed (my workgroup << 4 | 15) names my segment and where
+    // it starts, at one scalar compare and one scalar select per entry.
+    const uint32_t wg = blockIdx.x;
+    const uint32_t mine = (wg << 4) | 15u;
+    uint32_t best = a.first_wg[0];
+#pragma unroll
+    for (int k = 1; k < kMultiMaxSegments; ++k) {
+        const uint32_t f = a.first_wg[k];
+        best = f <= mine ? f : best;
+    }
+    const uint32_t s = best & 15u, base = best >> 4;
+    // The record is read through the kernel-argument pointer at a computed offset, so that the
+    // dynamic index turns into an address and not into a private copy of the table.
+    const KernargBytes ka = (KernargBytes)__builtin_amdgcn_kernarg_segment_ptr();
+    typedef const AdamSegment __attribute__((address_space(4))) * SegPtr;
+    const SegPtr sg = reinterpret_cast<SegPtr>(ka + __builtin_offsetof(AdamMultiArgs, seg) + s * sizeof(AdamSegment));
+    AdamConsts c;
+    c.beta1 = sg->c.beta1;
+    c.beta2 = sg->c.beta2;
+    c.omb1 = sg->c.omb1;
+    c.omb2 = sg->c.omb2;
+    c.bias2 = sg->c.bias2;
+    c.eps = sg->c.eps;
+    c.step_size = sg->c.step_size;
+    c.wd_coef = sg->c.wd_coef;
+    c.grad_mult = sg->c.grad_mult;
+    c.wd_mode = sg->c.wd_mode;
+    if constexpr (HAS_CTL) {
+        if (a.ctl->skip) return;
+        c.grad_mult = a.ctl->grad_mult;
+    }
+    const uint32_t local = wg - base;
+    const uint32_t head = sg->head, body_tiles = sg->body_tiles;
+    float* const p = sg->p;
+    float* const m = sg->m;
+    float* const v = sg->v;
+    const char* const g = static_cast<const char*>(sg->g);
+    char* const h = static_cast<char*>(sg->h);
+    constexpr uint32_t gsz = (GT == FT_F32) ? 4 : 2;
+    if (local < body_tiles) {
+        const uint64_t t0 = (uint64_t)local * kWave;  // first unit of the tile behind the head
+        const uint64_t i = t0 + threadIdx.x;
+        f32x4 g4 = load_g4<GT, true>(g + (uint64_t)head * gsz, i);
+        f32x4 p4 = ld<true>(reinterpret_cast<const f32x4*>(p + head) + i);
+        f32x4 m4 = ld<true>(reinterpret_cast<const f32x4*>(m + head) + i);
+        f32x4 v4 = ld<true>(reinterpret_cast<const f32x4*>(v + head) + i);
+        adam_unit(p4, g4, m4, v4, c);
+        const __amdgpu_buffer_rsrc_t rp = tile_rsrc(reinterpret_cast<f32x4*>(p + head) + t0, kWave * 16),
+                                     rm = tile_rsrc(reinterpret_cast<f32x4*>(m + head) + t0, kWave * 16),
+                                     rv = tile_rsrc(reinterpret_cast<f32x4*>(v + head) + t0, kWave * 16);
+        st_stream(rp, threadIdx.x * 16, p4);
+        st_stream(rm, threadIdx.x * 16, m4);
+        st_stream(rv, threadIdx.x * 16, v4);
+        if constexpr (HT == FT_F16 || HT == FT_BF16) {
+            const __amdgpu_buffer_rsrc_t rh = tile_rsrc(reinterpret_cast<u32x2*>(h + (uint64_t)head * 2) + t0, kWave * 8);
+            u32x2 w;
+            w.x = pack2<HT>(p4.x, p4.y);
+            w.y = pack2<HT>(p4.z, p4.w);
+            st_stream(rh, threadIdx.x * 8, w);
+        }
+        return;
+    }
+    // edge workgroup of the segment
+    const uint64_t n = sg->n;
+    const uint64_t tail0 = head + (uint64_t)body_tiles * (kWave * 4);
+    const uint32_t edge = head + (uint32_t)(n - tail0);
+    for (uint32_t e = threadIdx.x; e < edge; e += kWave) {
+        const uint64_t i = e < head ? e : tail0 + (e - head);
+        float gi;
+        if constexpr (GT == FT_F32)
+            gi = reinterpret_cast<const float*>(g)[i];
+        else
+            gi = half_to_float<GT>(reinterpret_cast<const uint16_t*>(g)[i]);
+        float pi = p[i], mi = m[i], vi = v[i];
+        adam_element(pi, gi, mi, vi, c);
+        p[i] = pi;
+        m[i] = mi;
+        v[i] = vi;
+        if constexpr (HT == FT_F16 || HT == FT_BF16)
+            reinterpret_cast<uint16_t*>(h)[i] = (uint16_t)(pack2<HT>(pi, 0.0f) & 0xffffu);
+    }
+}
+
 // ---- reductions ----------------------------------------------------------------------------
 // Sum across the 64 lanes of a wavefront with DPP lane permutes (no LDS): xor-1 and xor-2 inside
 // each quad, then mirror inside half rows and rows; every lane of a 16-lane row then holds the

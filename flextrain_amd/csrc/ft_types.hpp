@@ -30,4 +30,31 @@ struct AdamArgs {
     AdamConsts c;
 };
 
+// ---- many segments in one launch -------------------------------------------------------------
+// One contiguous piece of an in-place update with its own hyper-parameters: what the reference
+// hands to one adam_update call per StepContext (flextrain/optimizer.py:44-69).
+constexpr int kMultiMaxSegments = 16;
+
+struct AdamSegment {
+    float* p;
+    const void* g;
+    float* m;
+    float* v;
+    void* h;              // low-precision copy of this segment, or nullptr for every segment of a launch
+    uint64_t n;           // elements
+    uint32_t head;        // elements in front of the first tile (they reach the alignment the tiles want)
+    uint32_t body_tiles;  // whole 256-element tiles behind the head
+    AdamConsts c;
+};
+
+// The whole table travels in the kernel-argument segment (1.6 KB): no device allocation, no upload.
+// first_wg[s] = (number of workgroups that belong to the segments before s) << 4 | s; unused
+// entries hold 0xffffffff. A launch therefore has fewer than 2^28 workgroups.
+constexpr unsigned kMultiMaxWorkgroups = (1u << 28) - 1;
+struct AdamMultiArgs {
+    uint32_t first_wg[kMultiMaxSegments];
+    const ft_step_control_t* ctl;
+    AdamSegment seg[kMultiMaxSegments];
+};
+
 }  // namespace ftk

@@ -99,6 +99,17 @@ class FlexTrainCPUOptimizer(ABC):
         return guard.read() if guard is not None else None
 
     def _step_all(self, step_contexts: List[StepContext], extensions) -> None:
+        """One native call per context as in the reference's loop -- unless the engine can take
+        several resident contexts in one launch (``_step_many``) and there is more than one."""
+        many = getattr(self, "_step_many", None)
+        if many is not None and len(step_contexts) > 1:
+            live = [ctx for ctx in step_contexts if ctx.gradient.numel()]
+            resident = [ctx for ctx in live if ctx.full_parameter.is_cuda]
+            if len(resident) > 1 and len({(c.full_parameter.device, c.gradient.dtype) for c in resident}) == 1 \
+                    and len({c.half_parameter.dtype for c in resident if c.half_parameter is not None}) <= 1 \
+                    and set(extensions) <= {"grad_mult", "control", "blocking", "guard_stream"}:
+                many(resident, grad_mult=extensions.get("grad_mult", 1.0), control=extensions.get("control"))
+                step_contexts = [ctx for ctx in live if not ctx.full_parameter.is_cuda]
         for ctx in step_contexts:
             if not ctx.gradient.numel():
                 continue

@@ -87,6 +87,32 @@ int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, floa
                  int g_dtype, void* m, void* v, void* half_out, int half_dtype, size_t n,
                  const void* ctl, void* stream);
 
+/* ---- many resident updates in one launch -------------------------------------------------------
+ * Replaces the loop of flextrain/optimizer.py:44-69 (one adam_update[_copy] call per StepContext;
+ * flextrain/param_group.py:365-477 cuts a unit's share into one context per parameter group and
+ * buffer piece, each with its own hyper-parameters and step count): every segment is what one
+ * ft_adam_step call would take, and up to 16 of them run as ONE kernel launch (more segments, or
+ * segments with and without a low-precision copy, are spread over a few launches). Results are
+ * those of ft_adam_step segment by segment, bit for bit. Segments must not overlap one another.
+ * A segment whose arrays do not share their alignment is stepped element by element by a launch
+ * of its own. In place, resident arrays only; g_dtype, half_dtype and ctl apply to all segments.
+ * Nothing is allocated, copied or synchronised: the segment table travels with the launch. */
+typedef struct ft_adam_segment_t {
+    void* p;            /* fp32 master parameters, updated in place                       */
+    const void* g;      /* gradients (g_dtype)                                             */
+    void* m;            /* exp_avg                                                         */
+    void* v;            /* exp_avg_sq                                                      */
+    void* half_out;     /* NULL or the low-precision copy (half_dtype)                     */
+    size_t n;           /* elements; 0 = nothing to do                                     */
+    uint64_t step;
+    float lr, beta1, beta2, eps, weight_decay;
+    int32_t bias_correction;
+    float grad_mult;
+    int32_t reserved;   /* 0 */
+} ft_adam_segment_t;
+int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_dtype, int half_dtype,
+                       const void* ctl, void* stream);
+
 /* ---- gradient statistics and the skip / clip decision -----------------------------------
  * No counterpart in the reference: it scales the loss (flextrain/engine.py:249) but never
  * unscales, checks or clips gradients, and nothing calls DynamicLossScaler.update_scale
