@@ -357,6 +357,33 @@ int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need
 
 constexpr int kReduceBlocks = 256;  // second-level blocks of the accumulation pass's statistics
 
+// Statistics scratch of ft_grad_accumulate_static: block partials followed by one wavefront partial
+// per 256 elements, for calls of up to FT_STATIC_MAX_ELEMS elements. It is part of the loaded code
+// object, so every GPU the library runs on holds its own copy (8.1 MiB) until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress, never an address.
+constexpr size_t kStaticScratchBytes =
+    sizeof(ftk::StatsPartial) * kMaxStatsBlocks + (static_cast<size_t>(FT_STATIC_MAX_ELEMS) / 256 + 1) * sizeof(ftk::WavePartial);
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+
+std::unordered_map<int, void*> g_static_scratch_ptr;  // device -> that device's copy of the array
+
+// The current device's address of the array; looked up once per device, with that device current.
+int static_scratch(void** out)
+{
+    int dev = 0;
+    FT_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_static_scratch_ptr.find(dev);
+    if (it == g_static_scratch_ptr.end()) {
+        void* ptr = nullptr;
+        FT_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch)));
+        if (!ptr) return fth::fail(FT_EHIP, "hipGetSymbolAddress returned a null address for the statistics scratch");
+        it = g_static_scratch_ptr.emplace(dev, ptr).first;
+    }
+    *out = it->second;
+    return FT_OK;
+}
+
 // Wavefront partials of the accumulation pass live behind the fixed block-partial area.
 size_t accumulate_workspace_bytes(size_t n)
 {
@@ -640,9 +667,15 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
     return FT_OK;
 }
 
-int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
-                       float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
-                       size_t workspace_bytes, void* stream_)
+}  // extern "C"
+
+namespace {
+
+// static_scratch_only: the statistics scratch is the library's static device array (nothing is
+// allocated); otherwise the caller's workspace, or the library-owned buffer when that is NULL.
+int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                         float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
+                         size_t workspace_bytes, bool static_scratch_only, void* stream_)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (!valid_dtype(acc_dtype) || !valid_dtype(g_dtype))
@@ -661,7 +694,12 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
         nvec = (n - head) / 4;
     }
     ftk::StatsPartial* parts = nullptr;
-    if (stats) {
+    if (stats && static_scratch_only) {
+        void* ptr = nullptr;
+        int wrc = static_scratch(&ptr);
+        if (wrc != FT_OK) return wrc;
+        parts = static_cast<ftk::StatsPartial*>(ptr);
+    } else if (stats) {
         int wrc = resolve_stats_workspace(workspace, workspace_bytes, accumulate_workspace_bytes(n), &parts);
         if (wrc != FT_OK) return wrc;
     }
@@ -671,6 +709,29 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
         case FT_F16: return launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
         default: return launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
     }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                       float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
+                       size_t workspace_bytes, void* stream)
+{
+    return grad_accumulate_impl(acc, acc_dtype, g, g_dtype, n, scale, zero_g, stats_pre_mult, stats_out, stats_accumulate,
+                                workspace, workspace_bytes, false, stream);
+}
+
+int ft_grad_accumulate_static(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                              float stats_pre_mult, void* stats_out, int stats_accumulate, void* stream)
+{
+    if (n > static_cast<size_t>(FT_STATIC_MAX_ELEMS))
+        return fth::fail(FT_EINVAL, "ft_grad_accumulate_static takes at most %llu elements per call, got %zu "
+                         "(use ft_grad_accumulate with a workspace for longer buffers)",
+                         static_cast<unsigned long long>(FT_STATIC_MAX_ELEMS), n);
+    return grad_accumulate_impl(acc, acc_dtype, g, g_dtype, n, scale, zero_g, stats_pre_mult, stats_out, stats_accumulate,
+                                nullptr, 0, true, stream);
 }
 
 int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ctl_out, void* stream)

@@ -144,6 +144,18 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
                        float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/* ft_grad_accumulate_static: ft_grad_accumulate for callers that cannot allocate (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc). No counterpart in the
+ * reference. Same arguments, results and kernels as ft_grad_accumulate, without the workspace: the
+ * statistics scratch is a static device array inside the library (about 8.1 MiB on every GPU the
+ * library runs on, held until the process ends), so the call allocates and frees nothing, whatever
+ * the size of earlier calls. At most FT_STATIC_MAX_ELEMS elements per call (FT_EINVAL beyond).
+ * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two
+ * threads) race on it and must be ordered by the caller. */
+#define FT_STATIC_MAX_ELEMS (1ull << 28)
+int ft_grad_accumulate_static(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                              float stats_pre_mult, void* stats_out, int stats_accumulate, void* stream);
+
 /* ft_grad_control: turns statistics into the per-step decision, on the device:
  *   skip      = stats->nonfinite != 0
  *   norm      = sqrt(stats->sumsq)                                (double)
