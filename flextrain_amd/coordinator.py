@@ -27,8 +27,28 @@ What changes because the optimizer runs on the GPU:
     part, ``coordinator/parameter.py:470-519``) gets each element's new value in the piece that
     holds it, written over the link by the same step.
 Left out (other subsystems): the forward/backward alpha split with borrowed buffers, the NVMe
-tier, gradient reduce-scatter across ranks. Global-norm clipping cannot be combined with
-stepping during backward (the norm is known only after the last unit) and is not offered here.
+tier, gradient reduce-scatter across ranks.
+
+Mixed precision. The reference scales the loss (``flextrain/engine.py:249``) and never unscales
+(``flextrain/loss_scaler.py:134-179`` is a state machine nobody drives). With ``loss_scaler=`` every
+share's update multiplies its gradients by ``1/loss_scale`` on load, every unit's finished
+gradients are checked for inf/nan (for free where the fused accumulation pass runs anyway, else one
+read of the gradients) into ONE device-side record per iteration, and ``clear_backward_pipeline()``
+returns the iteration's ``GuardDecision`` and drives ``update_scale``. Two schedules:
+
+  * stepping during backward (default): a unit is stepped before the units in front of it have
+    produced their gradients, so the decision cannot be global. A unit is skipped (by its kernels,
+    on the device, no host round trip) when an inf/nan has been seen in its own gradients or in
+    those of any unit that finished before it in this iteration; units already stepped keep their
+    update; the iteration counts as overflowed and the scale goes down. Clipping by the global
+    norm is impossible here and refused.
+  * ``defer_to_forward=True``: backward only accumulates and gathers statistics, every unit keeps
+    its gradients in HBM (27 GB for a 7B model in bf16: what 288 GB are for), the decision is taken
+    once after the first unit's backward -- skip everything or nothing, one clip coefficient from
+    the norm over ALL units -- and unit ``u+1`` is stepped share by share during the next
+    iteration's forward pass of unit ``u`` (``warmup_forward_pipeline``, ``pre_unit_forward``,
+    ``post_micro_batch_forward``: the forward-side hooks of the reference, ``:758-769,784-794,
+    825-847``, which there step the forward share of the alpha split).
 """
 from __future__ import annotations
 
@@ -72,6 +92,10 @@ class FlexTrainOptsCoordinator:
         offload: bool = True,
         unit_windows: Optional[bool] = None,
         window_write_through: bool = False,
+        loss_scaler=None,
+        check_overflow: Optional[bool] = None,
+        max_grad_norm: Optional[float] = None,
+        defer_to_forward: bool = False,
     ) -> None:
         """
         Args:
@@ -100,6 +124,15 @@ class FlexTrainOptsCoordinator:
             window_write_through: a window's results are written to the host by the step kernels
                 themselves instead of being copied back in one piece after the unit's last share
                 (slower: 43.7 GB/s on the same schedule).
+            loss_scaler: object with ``loss_scale`` and ``update_scale(overflow)``
+                (``flextrain_amd.loss_scaler``): the gradients were produced from
+                ``loss * loss_scale`` and are divided by it inside the update.
+            check_overflow: look for inf/nan in every unit's gradients and skip on the device
+                (default: on when a loss scaler is given).
+            max_grad_norm: clip the L2 norm of the unscaled gradients of all units together to this
+                value; needs ``defer_to_forward``.
+            defer_to_forward: keep every unit's gradients and step during the next forward pass,
+                after one global decision (see the module docstring).
         """
         units = [[u] if isinstance(u, Tensor) else list(u) for u in unit_half_parameters]
         assert units and all(units)
@@ -134,11 +167,38 @@ class FlexTrainOptsCoordinator:
             raise NotImplementedError("units must hold fp16 or bf16 parameters; the fp32 master copy is kept beside them")
         gradacc_dtype = gradacc_dtype or device_dtype
         self._gradacc_dtype_incompatible = gradacc_dtype != device_dtype
+        self._device = device
 
-        # Two gradient buffers trade places every unit: [0] receives the unit in backward,
-        # [1] holds the finished gradients of the unit being stepped.
+        self._loss_scaler = loss_scaler
+        self._check_overflow = bool(loss_scaler is not None if check_overflow is None else check_overflow)
+        self._max_grad_norm = float(max_grad_norm) if max_grad_norm else None
+        self._defer = bool(defer_to_forward)
+        if self._max_grad_norm is not None and not self._defer:
+            raise ValueError("clipping by the global norm needs every unit's gradients before the first update: "
+                             "use defer_to_forward=True")
+        self._guarded = self._check_overflow or self._max_grad_norm is not None
+        self._iter_guard = None       # the iteration's statistics record and scratch
+        self._unit_controls = None    # one ft_step_control_t per unit (row u), 16 bytes each
+        self._iteration_open = False  # statistics of the running iteration have been started
+        self._pending_steps = False   # deferred schedule: a decision has been taken and not yet applied
+        self._deferred_skip = False
+        self.last_decision = None
+        self.last_skipped_units: List[int] = []
+        if self._guarded:
+            from .loss_scaler import GradientGuard
+            self._iter_guard = GradientGuard(device)
+            self._unit_controls = torch.zeros(self._num_units + 1, 4, dtype=torch.float32, device=device)
+            self._unit_controls[:, 1] = 1.0
+            self._unit_controls[:, 3] = 1.0
+
+        # Stepping during backward: two gradient buffers trade places every unit, [0] receives the
+        # unit in backward, [1] holds the finished gradients of the unit being stepped. Deferred:
+        # every unit keeps a buffer of its own until its update, one iteration later.
         self._gpu_bwd_grad_buffers = RotateContainer(tuple(
-            allocate_memory_chunks(self._unit_numel, 2, gradacc_dtype, device)))
+            allocate_memory_chunks(self._unit_numel, 2, gradacc_dtype, device))) if not self._defer else None
+        self._unit_grads = allocate_memory_chunks(self._unit_numel, self._num_units, gradacc_dtype, device) \
+            if self._defer else None
+        self._bwd_unit = -1  # deferred: the unit whose backward is running
         # When gradients are accumulated in a wider type than backward produces them in, backward
         # writes each micro-batch into this extra buffer and one fused pass per micro-batch adds it
         # to the receive buffer and clears it (reference ``:187-190,743,775-777``: a zero_ before
@@ -147,7 +207,7 @@ class FlexTrainOptsCoordinator:
         if self._gradacc_dtype_incompatible:
             from .loss_scaler import GradientGuard
             self._gpu_bwd_extra_grads = allocate_memory_chunks(self._unit_numel, 1, device_dtype, device)[0]
-            self._guard = GradientGuard(device)
+            self._guard = self._iter_guard if self._iter_guard is not None else GradientGuard(device)
 
         # [master | exp_avg | exp_avg_sq] per unit.
         per_element = 1 + optimizer.optimizer_state_per_element
@@ -185,11 +245,16 @@ class FlexTrainOptsCoordinator:
     # ---- buffers -------------------------------------------------------------------------------
     @property
     def _gpu_bwd_receive_grads(self) -> Tensor:
-        return self._gpu_bwd_grad_buffers[0]
+        return self._unit_grads[self._bwd_unit] if self._defer else self._gpu_bwd_grad_buffers[0]
 
     @property
     def _gpu_bwd_step_grads(self) -> Tensor:
         return self._gpu_bwd_grad_buffers[1]
+
+    @property
+    def loss_scale(self) -> float:
+        """What the training loop multiplies the loss by (reference ``flextrain/engine.py:249``)."""
+        return float(self._loss_scaler.loss_scale) if self._loss_scaler is not None else 1.0
 
     def unit_master_parameter(self, unit_index: int) -> Tensor:
         return self._unit_opts[unit_index][0]
@@ -198,19 +263,23 @@ class FlexTrainOptsCoordinator:
         return list(self._unit_opts[unit_index][1:])
 
     def _rotate_buffers(self) -> None:
-        self._gpu_bwd_grad_buffers.rotate()
+        if not self._defer:
+            self._gpu_bwd_grad_buffers.rotate()
 
     # ---- steps ---------------------------------------------------------------------------------
     def _plan_optimizer_steps(self, unit_index: int, execute_now: bool = False) -> None:
         """Bind the unit's step contexts to its buffers (reference ``:605-682``)."""
         if self._is_invalid_unit(unit_index):
             return
+        if self._defer and self._deferred_skip:
+            return  # the whole iteration is skipped: nothing to bind, nothing to bring to the GPU
         self._unit_step_ctxts[unit_index].plan(
             half_parameter=self._unit_half_parameters[unit_index],
             full_parameter=self._unit_opts[unit_index][0],
-            gradient=self._gpu_bwd_step_grads,
+            gradient=self._unit_grads[unit_index] if self._defer else self._gpu_bwd_step_grads,
             optimizer_states=[[s] for s in self._unit_opts[unit_index][1:]],
         )
+        self._decide_unit(unit_index)
         self._open_unit_window(unit_index)
         if execute_now:
             for mb in range(self._micro_batch_per_rank):
@@ -220,6 +289,8 @@ class FlexTrainOptsCoordinator:
         """Starts bringing a unit's master state to the GPU (no-op without windows, for an invalid
         unit, or when it is already on its way). Called one unit ahead of the unit's steps, so the
         copies run while the previous unit is still being stepped."""
+        if self._defer and self._deferred_skip:
+            return
         if self._unit_windows and not self._is_invalid_unit(unit_index) and unit_index not in self._open_windows:
             self._open_windows[unit_index] = self._optimizer.cpu_optimizer.open_window(*self._unit_opts[unit_index], write_through=self._window_write_through)
 
@@ -228,13 +299,64 @@ class FlexTrainOptsCoordinator:
         work is enqueued."""
         if self._is_invalid_task(unit_index, micro_batch_index):
             return
+        if self._defer and self._deferred_skip:
+            return
         contexts = self._unit_step_ctxts[unit_index][micro_batch_index]
+        extensions = {}
+        if self._guarded:  # skip and the gradient multiplier come from the unit's device-side record
+            extensions["control"] = self._unit_controls[self._num_units if self._defer else unit_index]
+        elif self._loss_scaler is not None:
+            extensions["grad_mult"] = float(1.0 / self.loss_scale)
         if self._offload:
-            self._optimizer.cpu_optimizer.step(contexts, blocking=False, guard_stream=False)
+            self._optimizer.cpu_optimizer.step(contexts, blocking=False, guard_stream=False, **extensions)
             if micro_batch_index == self._micro_batch_per_rank - 1 and unit_index in self._open_windows:
                 self._optimizer.cpu_optimizer.close_window(self._open_windows.pop(unit_index))
         else:
-            self._optimizer.cpu_optimizer.step(contexts)
+            self._optimizer.cpu_optimizer.step(contexts, **extensions)
+
+    # ---- statistics and decisions ---------------------------------------------------------------
+    def _begin_iteration_statistics(self) -> None:
+        if self._guarded and not self._iteration_open:
+            self._iter_guard.begin()
+            self._iteration_open = True
+
+    def _gather_unit_statistics(self, grads: Tensor) -> None:
+        """Adds one finished unit's gradients to the iteration's record -- unless the fused
+        accumulation pass of its last micro-batch has done so already."""
+        if self._guarded and not self._gradacc_dtype_incompatible:
+            self._iter_guard.add(grads, loss_scale=self.loss_scale)
+
+    def _decide_unit(self, unit_index: int) -> None:
+        """Stepping during backward: the unit's control record from everything seen so far in this
+        iteration (its own gradients and those of the units that finished before it)."""
+        if not self._guarded or self._defer:
+            return
+        self._gather_unit_statistics(self._gpu_bwd_step_grads)
+        self._iter_guard.decide_async(loss_scale=self.loss_scale, out=self._unit_controls[unit_index])
+
+    def _finish_iteration_statistics(self):
+        """Reads the iteration's record back (one small copy), drives the loss scaler and returns the
+        ``GuardDecision``; None when nothing is checked."""
+        if not self._guarded:
+            return None
+        from .loss_scaler import GuardDecision
+        stats = self._iter_guard._buf[:2].cpu()  # waits for the stream: every statistics pass has run
+        controls = self._unit_controls.cpu()
+        nonfinite = int(stats[0:1].view(torch.int64).item())
+        final = controls[self._num_units if self._defer else 0]  # the record that saw every unit
+        skipped = (controls[:, 0].contiguous().view(torch.int32) != 0).tolist()
+        if self._defer:
+            self.last_skipped_units = list(range(self._num_units)) if skipped[self._num_units] else []
+        else:
+            self.last_skipped_units = [u for u in range(self._num_units) if skipped[u]]
+        decision = GuardDecision(overflow=nonfinite != 0, nonfinite=nonfinite, sumsq=float(stats[1].item()),
+                                 grad_norm=float(final[2].item()), clip_coef=float(final[3].item()),
+                                 grad_mult=float(final[1].item()))
+        self.last_decision = decision
+        self._iteration_open = False
+        if self._loss_scaler is not None:
+            self._loss_scaler.update_scale(decision.overflow)
+        return decision
 
     # ---- hooks of the training loop ------------------------------------------------------------
     def pre_unit_backward(self, unit_index: int) -> Tensor:
@@ -242,30 +364,104 @@ class FlexTrainOptsCoordinator:
         Returns the zeroed buffer backward must write the unit's gradients into: the accumulation
         buffer itself (backward accumulates over micro-batches), or -- when accumulation happens in
         a wider type -- the buffer for one micro-batch's gradients."""
+        if self._defer and self._pending_steps:
+            raise RuntimeError("the previous iteration's updates have not been applied: run the forward-side hooks "
+                               "(warmup_forward_pipeline, pre_unit_forward, post_micro_batch_forward) for every unit first")
+        self._begin_iteration_statistics()
         self._rotate_buffers()
         if self._offload:
-            # The buffer that now receives gradients fed the step of unit_index + 2; its kernels
-            # must have read it before backward overwrites it. A wait on the device, not the host.
+            # The buffer that now receives gradients fed a step enqueued earlier (of unit_index + 2,
+            # or, deferred, of this unit in the forward pass); its kernels must have read it before
+            # backward overwrites it. A wait on the device, not the host.
             self._optimizer.cpu_optimizer.stream_wait()
-        self._plan_optimizer_steps(unit_index + 1)
-        self._open_unit_window(unit_index)  # prefetch for the steps that start one unit from now
+        if self._defer:
+            self._bwd_unit = unit_index
+        else:
+            self._plan_optimizer_steps(unit_index + 1)
+            self._open_unit_window(unit_index)  # prefetch for the steps that start one unit from now
         receive = self._gpu_bwd_receive_grads
         receive.zero_()
         return self._gpu_bwd_extra_grads if self._gradacc_dtype_incompatible else receive
 
     def post_micro_batch_backward(self, unit_index: int, micro_batch_index: int) -> None:
         """Called after each micro-batch's backward of ``unit_index``: folds the micro-batch's
-        gradients into the accumulation buffer when the two differ in type, then steps the same
-        share of the unit that finished before it."""
+        gradients into the accumulation buffer when the two differ in type (the last micro-batch's
+        pass also yields the unit's overflow statistics), then steps the same share of the unit
+        that finished before it -- or, deferred, only gathers the finished unit's statistics."""
+        last = micro_batch_index == self._micro_batch_per_rank - 1
         if self._gradacc_dtype_incompatible:
-            self._guard.accumulate(self._gpu_bwd_receive_grads, self._gpu_bwd_extra_grads, zero_grads=True)
+            self._guard.accumulate(self._gpu_bwd_receive_grads, self._gpu_bwd_extra_grads, zero_grads=True,
+                                   with_stats=self._guarded and last, loss_scale=self.loss_scale)
+        if self._defer:
+            if last:
+                self._gather_unit_statistics(self._unit_grads[unit_index])
+            return
         self._execute_optimizer_step(unit_index + 1, micro_batch_index)
 
-    def clear_backward_pipeline(self) -> None:
-        """After the first unit's backward: step it, then wait for everything in flight."""
+    def clear_backward_pipeline(self):
+        """After the first unit's backward. Stepping during backward: step that unit, then wait for
+        everything in flight. Deferred: take the iteration's one decision (skip, clip coefficient)
+        on the device; the updates follow in the next forward pass. Returns the iteration's
+        ``GuardDecision`` (None when neither overflow checking nor clipping is on) after handing its
+        overflow flag to the loss scaler."""
+        if self._defer:
+            if self._guarded:
+                self._iter_guard.decide_async(loss_scale=self.loss_scale, max_grad_norm=self._max_grad_norm,
+                                              out=self._unit_controls[self._num_units])
+            decision = self._finish_iteration_statistics()
+            self._pending_steps = True
+            self._deferred_skip = bool(decision.overflow) if decision is not None else False
+            return decision
         self._rotate_buffers()
         self._plan_optimizer_steps(0, execute_now=True)
+        decision = self._finish_iteration_statistics()
         self.synchronize()
+        return decision
+
+    # ---- forward-side hooks (deferred schedule) --------------------------------------------------
+    def warmup_forward_pipeline(self) -> None:
+        """Before the forward pass of the first unit (reference ``:825-847``): its parameters must be
+        the updated ones, so its whole update is enqueued now; the second unit's state starts on its
+        way to the GPU. No-op unless a deferred decision is waiting to be applied. The caller
+        advances the groups' step counters (``update_states``) before this call when the decision
+        was not an overflow."""
+        if not (self._defer and self._pending_steps):
+            return
+        self._plan_optimizer_steps(0, execute_now=True)
+        self._open_unit_window(1)
+        self._fwd_guard_parameters()
+        if self._num_units == 1:
+            self._finish_deferred_steps()
+
+    def pre_unit_forward(self, unit_index: int) -> None:
+        """Before the forward pass of ``unit_index`` (reference ``:758-769``): bind the next unit's
+        step contexts and start prefetching the state of the one after it."""
+        if not (self._defer and self._pending_steps):
+            return
+        self._plan_optimizer_steps(unit_index + 1)
+        self._open_unit_window(unit_index + 2)
+
+    def post_micro_batch_forward(self, unit_index: int, micro_batch_index: int) -> None:
+        """After each micro-batch's forward of ``unit_index`` (reference ``:784-794``): step the same
+        share of the next unit; after the last share the next unit's forward may read its new
+        parameters."""
+        if not (self._defer and self._pending_steps):
+            return
+        self._execute_optimizer_step(unit_index + 1, micro_batch_index)
+        if micro_batch_index == self._micro_batch_per_rank - 1:
+            self._fwd_guard_parameters()
+            if unit_index + 1 >= self._num_units - 1:
+                self._finish_deferred_steps()
+
+    def _fwd_guard_parameters(self) -> None:
+        """The forward pass that follows on the caller's stream reads the low-precision parameters the
+        offloaded step's kernels (on the engine's stream) have just written."""
+        if self._offload and not self._deferred_skip:
+            self._optimizer.cpu_optimizer.stream_wait()
+
+    def _finish_deferred_steps(self) -> None:
+        self._pending_steps = False
+        self._deferred_skip = False
 
     def synchronize(self) -> None:
         if self._offload:

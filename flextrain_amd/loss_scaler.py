@@ -223,15 +223,22 @@ class GradientGuard:
         if with_stats:
             self._fresh = False
 
-    def decide_async(self, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None) -> torch.Tensor:
+    def decide_async(self, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Turns the statistics gathered so far into a control record on the device and returns it
+        (the guard's own record, or ``out``: 16 bytes of device memory, 16-byte aligned, for callers
+        that keep one record per unit of work)."""
         if self._fresh:
             raise RuntimeError("decide() before any add()")
         inv_scale = float(1.0 / float(loss_scale))
+        target = self.control if out is None else out
+        if out is not None and (not out.is_cuda or out.numel() * out.element_size() < 16 or out.data_ptr() % 16):
+            raise ValueError("out must be 16 bytes of 16-byte aligned device memory")
         with torch.cuda.device(self.device):
             _C.check("ft_grad_control", self._lib.ft_grad_control(
                 self.stats_ptr, inv_scale, float(max_grad_norm) if max_grad_norm else 0.0,
-                self.control.data_ptr(), _C.current_stream_ptr(self.device)))
-        return self.control
+                target.data_ptr(), _C.current_stream_ptr(self.device)))
+        return target
 
     def decide(self, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None) -> GuardDecision:
         self.decide_async(loss_scale, max_grad_norm)

@@ -206,3 +206,174 @@ def test_state_files_resume_bit_exact(cuda, tmp_path, offload):
         assert torch.equal(coord_a.unit_master_parameter(u).cpu(), coord_b.unit_master_parameter(u).cpu())
         for sa, sb in zip(coord_a.unit_optimizer_states(u), coord_b.unit_optimizer_states(u)):
             assert torch.equal(sa.cpu(), sb.cpu())
+
+
+# ---- mixed precision in the per-unit pipeline ---------------------------------------------------
+def _fp16_units(cuda, num_units, unit_numel, offload, **coordinator_kwargs):
+    from flextrain_amd import FlexTrainAdam
+    from flextrain_amd.coordinator import FlexTrainOptsCoordinator
+    flat = [(torch.randn(unit_numel, device=cuda) * 0.02).to(torch.float16) for _ in range(num_units)]
+    params = [torch.nn.Parameter(f) for f in flat]
+    group = {"params": params, "weight_decay": 0.01}
+    opt = FlexTrainAdam([group], lr=1e-3, unit_parameter_map={u: _Unit([params[u]]) for u in range(num_units)},
+                        aligned_unit_numel=unit_numel, offload=offload)
+    coord = FlexTrainOptsCoordinator()
+    coord.initialize(opt, flat, offload=offload, device=cuda, **coordinator_kwargs)
+    state = [(to_np(flat[u].float()).copy(), np.zeros(unit_numel, np.float32), np.zeros(unit_numel, np.float32))
+             for u in range(num_units)]
+    return flat, group, opt, coord, state
+
+
+def _check_units(tag, coord, flat, state, expected_half):
+    for u, (pn, mn, vn) in enumerate(state):
+        m, v = coord.unit_optimizer_states(u)
+        worst = dict(p=max_ulp(to_np(coord.unit_master_parameter(u)), pn), m=max_ulp(to_np(m), mn), v=max_ulp(to_np(v), vn),
+                     h=max_ulp(half_bits(flat[u]).view(np.float16), expected_half[u].view(np.float16)))
+        print(f"[{tag} unit={u}] worst ULP distance: {worst}", flush=True)
+        assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst["h"] <= HALF_ULP, (tag, u, worst)
+
+
+@pytest.mark.parametrize("offload,windows,gradacc", [(False, False, None), (True, True, None), (True, False, None),
+                                                     (False, False, torch.float32), (True, True, torch.float32)])
+def test_scaled_gradients_and_overflow_while_stepping_during_backward(cuda, oracle, offload, windows, gradacc):
+    """fp16 units, loss scale 65536, three iterations, an inf planted in unit 1 on iteration 2.
+    Every share's update unscales on load; the policy for an overflow found after earlier units have
+    been stepped: unit 1 and every unit stepped after it (unit 0) are skipped on the device, units 3
+    and 2 keep their update, the iteration is flagged and the scale halves. State of every unit
+    against the oracle under that policy; scale trace against the reference's state machine."""
+    from flextrain_amd.loss_scaler import DynamicLossScaler
+    torch.manual_seed(5)
+    num_units, micro_batches, unit_numel = 4, 2, 1 << 18
+    scaler = DynamicLossScaler(init_scale=65536.0, delayed_shift=1, scale_window=1000)
+    flat, group, opt, coord, state = _fp16_units(
+        cuda, num_units, unit_numel, offload, micro_batch_per_rank=micro_batches, unit_windows=windows,
+        gradacc_dtype=gradacc, loss_scaler=scaler)
+    expected_half = [half_bits(f).copy() for f in flat]
+    gen = torch.Generator(device=cuda).manual_seed(9)
+    seen_scales, overflows = [], []
+    for iteration in (1, 2, 3):
+        scale = coord.loss_scale
+        seen_scales.append(scale)
+        opt.update_states()
+        accumulated = {}
+        for u in reversed(range(num_units)):
+            buf = coord.pre_unit_backward(u)
+            acc = np.zeros(unit_numel, np.float32) if gradacc is not None else None
+            for mb in range(micro_batches):
+                g = (torch.randn(unit_numel, device=cuda, generator=gen) * 1e-3 * scale).to(torch.float16)
+                if iteration == 2 and u == 1 and mb == 0:
+                    g[12345] = float("inf")
+                if gradacc is None:
+                    buf += g
+                else:
+                    buf.copy_(g)
+                    oracle.grad_accumulate(acc, CODE[torch.float32], half_bits(g).copy(), CODE[torch.float16])
+                if mb == micro_batches - 1:
+                    accumulated[u] = buf.clone() if gradacc is None else acc
+                coord.post_micro_batch_backward(u, mb)
+        decision = coord.clear_backward_pipeline()
+        overflows.append(decision.overflow)
+        assert decision.overflow == (iteration == 2) and decision.nonfinite == (1 if iteration == 2 else 0)
+        assert coord.last_skipped_units == ([0, 1] if iteration == 2 else [])
+        for u in range(num_units):
+            if iteration == 2 and u <= 1:
+                continue  # skipped: the oracle's state stays as it is
+            pn, mn, vn = state[u]
+            gn = accumulated[u] if gradacc is not None else half_bits(accumulated[u])
+            hn = np.zeros(unit_numel, np.uint16)
+            oracle.adam_step(pn, gn, mn, vn, step=iteration, lr=1e-3, weight_decay=0.01,
+                             grad_mult=float(np.float32(1.0 / scale)),
+                             g_dtype=CODE[torch.float32] if gradacc is not None else CODE[torch.float16],
+                             half_out=hn, half_dtype=CODE[torch.float16])
+            expected_half[u] = hn
+        _check_units(f"scaled offload={offload} windows={windows} gradacc={gradacc} it={iteration}", coord, flat, state, expected_half)
+    assert seen_scales + [coord.loss_scale] == oracle.loss_scale_trace(overflows, 65536.0, delayed_shift=1)
+    assert overflows == [False, True, False]
+
+
+@pytest.mark.parametrize("offload,windows,gradacc", [(False, False, None), (True, True, None), (True, False, torch.float32)])
+def test_deferred_schedule_gives_a_global_decision(cuda, oracle, offload, windows, gradacc):
+    """defer_to_forward: backward only accumulates and gathers statistics; one decision per
+    iteration after the first unit's backward; the updates run during the next forward pass.
+    Iteration 2 carries a nan in the LAST unit to run backward (unit 0): every unit, also those whose
+    gradients were complete long before, stays bit-unchanged. Iterations 1 and 3 are clipped with
+    the norm over all units (against float64: 1e-6), and the state equals the oracle's."""
+    from flextrain_amd.loss_scaler import DynamicLossScaler
+    torch.manual_seed(6)
+    num_units, micro_batches, unit_numel, max_norm = 3, 2, 1 << 18, 1.0
+    scaler = DynamicLossScaler(init_scale=4096.0, delayed_shift=1, scale_window=1000)
+    flat, group, opt, coord, state = _fp16_units(
+        cuda, num_units, unit_numel, offload, micro_batch_per_rank=micro_batches, unit_windows=windows,
+        gradacc_dtype=gradacc, loss_scaler=scaler, max_grad_norm=max_norm, defer_to_forward=True)
+    expected_half = [half_bits(f).copy() for f in flat]
+    gen = torch.Generator(device=cuda).manual_seed(10)
+
+    def forward_pass():
+        coord.warmup_forward_pipeline()
+        for u in range(num_units):
+            coord.pre_unit_forward(u)
+            for mb in range(micro_batches):
+                coord.post_micro_batch_forward(u, mb)
+
+    applied, seen_scales, overflows = 0, [], []
+    for iteration in (1, 2, 3):
+        forward_pass()  # applies the previous iteration's decision (nothing to apply in iteration 1)
+        coord.synchronize()
+        _check_units(f"deferred offload={offload} windows={windows} gradacc={gradacc} before it={iteration}", coord, flat, state, expected_half)
+        scale = coord.loss_scale
+        seen_scales.append(scale)
+        accumulated, sumsq = {}, 0.0
+        for u in reversed(range(num_units)):
+            buf = coord.pre_unit_backward(u)
+            acc = np.zeros(unit_numel, np.float32) if gradacc is not None else None
+            for mb in range(micro_batches):
+                g = (torch.randn(unit_numel, device=cuda, generator=gen) * 3e-3 * scale).to(torch.float16)
+                if iteration == 2 and u == 0 and mb == 1:
+                    g[777] = float("nan")
+                if gradacc is None:
+                    buf += g
+                else:
+                    buf.copy_(g)
+                    oracle.grad_accumulate(acc, CODE[torch.float32], half_bits(g).copy(), CODE[torch.float16])
+                if mb == micro_batches - 1:
+                    accumulated[u] = buf.clone() if gradacc is None else acc
+                coord.post_micro_batch_backward(u, mb)
+            unscaled = (accumulated[u].double() if gradacc is None else torch.from_numpy(acc).double()) / scale
+            sumsq += float((unscaled[torch.isfinite(unscaled)] ** 2).sum())
+        decision = coord.clear_backward_pipeline()
+        overflows.append(decision.overflow)
+        assert decision.overflow == (iteration == 2)
+        if decision.overflow:
+            assert coord.last_skipped_units == list(range(num_units))
+            continue
+        norm = sumsq ** 0.5
+        assert norm > max_norm and abs(decision.grad_norm - norm) <= 1e-6 * norm
+        assert abs(decision.clip_coef - max_norm / (norm + 1e-6)) <= 1e-6 * decision.clip_coef
+        assert np.float32(decision.grad_mult) == oracle.combined_multiplier(scale, decision.clip_coef)
+        applied += 1
+        opt.update_states()  # the caller advances the step counters of an iteration that will be applied
+        for u in range(num_units):
+            pn, mn, vn = state[u]
+            gn = accumulated[u] if gradacc is not None else half_bits(accumulated[u])
+            hn = np.zeros(unit_numel, np.uint16)
+            oracle.adam_step(pn, gn, mn, vn, step=applied, lr=1e-3, weight_decay=0.01, grad_mult=decision.grad_mult,
+                             g_dtype=CODE[torch.float32] if gradacc is not None else CODE[torch.float16],
+                             half_out=hn, half_dtype=CODE[torch.float16])
+            expected_half[u] = hn
+    with pytest.raises(RuntimeError, match="have not been applied"):
+        coord.pre_unit_backward(num_units - 1)
+    forward_pass()
+    coord.synchronize()
+    _check_units(f"deferred offload={offload} windows={windows} gradacc={gradacc} final", coord, flat, state, expected_half)
+    assert seen_scales + [coord.loss_scale] == oracle.loss_scale_trace(overflows, 4096.0, delayed_shift=1)
+    assert group["step"] == 2
+
+
+def test_clipping_needs_the_deferred_schedule(cuda):
+    from flextrain_amd import FlexTrainAdam
+    from flextrain_amd.coordinator import FlexTrainOptsCoordinator
+    flat = [torch.zeros(1024, dtype=torch.bfloat16, device=cuda)]
+    params = [torch.nn.Parameter(flat[0])]
+    opt = FlexTrainAdam([{"params": params}], unit_parameter_map={0: _Unit(params)}, aligned_unit_numel=1024, offload=False)
+    with pytest.raises(ValueError, match="defer_to_forward"):
+        FlexTrainOptsCoordinator().initialize(opt, flat, 2, offload=False, max_grad_norm=1.0)
