@@ -319,35 +319,52 @@ class FlexTrainOptimizer:
         """Steps the non-layerwise parameters (reference ``flextrain/optimizer.py:244-263``).
 
         Returns True if the update was applied, False if it was skipped because of inf/nan.
+        ``enqueue_step()`` followed by ``complete_step()``: nothing is read back from the GPU before
+        the update has been enqueued.
         """
+        self.enqueue_step()
+        return self.complete_step()
+
+    def enqueue_step(self) -> None:
+        """Everything of a step that runs on the GPU, enqueued on the current stream: statistics of
+        the gradients, the skip / unscale / clip decision (a 16-byte record that stays on the
+        device), the update reading that record, clearing the gradients. With resident state the
+        call does not wait for the GPU, allocates nothing after its first use and clears with
+        kernels, so a caller may record it into a HIP graph and replay it -- as long as the
+        hyper-parameters that travel by value (``group["step"]``, ``lr``, the loss scale) are meant
+        to stay what they were at capture. Offloaded state: the streamed update blocks until the
+        host arrays hold the new values, as the reference's host step does."""
         grads = self._step_grad
         if self._grad_reduce_fn is not None:
             self._grad_reduce_fn(grads)
-
         extensions = {}
-        self.last_step_skipped = False
-        if (self.loss_scaler is not None or self.max_grad_norm is not None) and grads.numel():
+        self._step_guarded = (self.loss_scaler is not None or self.max_grad_norm is not None) and grads.numel() > 0
+        if self._step_guarded:
             from .loss_scaler import GradientGuard  # local import: keeps module load light
             if not hasattr(self, "_guard"):
                 self._guard = GradientGuard(device=grads.device)
             scale = float(self.loss_scaler.loss_scale) if self.loss_scaler is not None else 1.0
             self._guard.begin()
             self._guard.add(grads, loss_scale=scale)
-            decision = self._guard.decide(loss_scale=scale, max_grad_norm=self.max_grad_norm)
-            self.last_grad_norm = decision.grad_norm
-            if self.loss_scaler is not None:
-                self.loss_scaler.update_scale(decision.overflow)
-            if decision.overflow:
-                self.last_step_skipped = True
-                self._zero_grads()
-                return False
-            extensions["grad_mult"] = decision.grad_mult
-
+            extensions["control"] = self._guard.decide_async(loss_scale=scale, max_grad_norm=self.max_grad_norm)
         self.cpu_optimizer.step(self.non_layerwise_step_contexts, **extensions)
         self._zero_grads()
         if self._offload and self._device_dtype == self._master_dtype:
             self._device_para.copy_(self._master_para, non_blocking=True)
-        return True
+
+    def complete_step(self) -> bool:
+        """Host side of a step, after ``enqueue_step()`` (or after replaying a graph that holds it):
+        reads the 32-byte statistics + decision record, hands the overflow flag to the loss scaler,
+        sets ``last_step_skipped`` / ``last_grad_norm``. Returns True if the update was applied."""
+        self.last_step_skipped = False
+        if not getattr(self, "_step_guarded", False):
+            return True
+        decision = self._guard.read()
+        self.last_grad_norm = decision.grad_norm
+        if self.loss_scaler is not None:
+            self.loss_scaler.update_scale(decision.overflow)
+        self.last_step_skipped = bool(decision.overflow)
+        return not decision.overflow
 
     def _zero_grads(self):
         self._device_grad.zero_()

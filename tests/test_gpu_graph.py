@@ -171,3 +171,56 @@ def test_gradient_hand_off_and_step_replay_in_a_hip_graph(cuda):
         eager_other = torch.randn(4099, device=cuda)  # unrelated eager work through the same library
         guards[id(twin)].begin(); guards[id(twin)].add(eager_other)
         torch.cuda.synchronize()
+
+
+def test_non_layerwise_step_replays_in_a_hip_graph(cuda):
+    """FlexTrainOptimizer.enqueue_step (statistics -> device-side decision -> update of every
+    parameter group in one launch -> clearing the gradients) recorded once and replayed, against a
+    twin optimizer stepped eagerly on the same gradients: same bits after every replay, also the
+    one whose gradients overflow. Static loss scale and a fixed step count: both travel by value."""
+    from flextrain_amd import FlexTrainAdam
+    from flextrain_amd.loss_scaler import LossScaler
+
+    def build():
+        torch.manual_seed(3)
+        a = torch.nn.Parameter((torch.randn(300, 257, device=cuda) * 0.02).to(torch.float16))
+        b = torch.nn.Parameter((torch.randn(1001, device=cuda) * 0.02).to(torch.float16))
+        c = torch.nn.Parameter((torch.randn(64, 64, device=cuda) * 0.02).to(torch.float16))
+        opt = FlexTrainAdam([{"params": [a, c], "weight_decay": 0.1}, {"params": [b], "weight_decay": 0.0, "lr": 3e-4}],
+                            lr=1e-3, loss_scaler=LossScaler(scale=1024.0), max_grad_norm=1.0)
+        opt.update_states()
+        return opt, (a, b, c)
+
+    eager, eager_params = build()
+    replayed, replay_params = build()
+    gen = torch.Generator(device=cuda).manual_seed(4)
+
+    def fresh_gradients(overflow):
+        for pe, pr in zip(eager_params, replay_params):
+            g = (torch.randn(pe.shape, device=cuda, generator=gen) * 0.3 * 1024.0).to(torch.float16)
+            if overflow and pe.dim() == 1:
+                g[17] = float("nan")
+            pe.grad.copy_(g)
+            pr.grad.copy_(g)
+
+    fresh_gradients(False)
+    assert eager.step() is True and replayed.step() is True  # warm-up: creates the guard and its scratch
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        replayed.enqueue_step()
+    torch.cuda.synchronize()
+    for replay, overflow in enumerate([False, True, False, False]):
+        fresh_gradients(overflow)
+        torch.cuda.synchronize()
+        graph.replay()
+        assert replayed.complete_step() is (not overflow)
+        assert eager.step() is (not overflow)
+        torch.cuda.synchronize()
+        assert replayed.last_grad_norm == eager.last_grad_norm or overflow
+        assert torch.equal(replayed._master_para, eager._master_para), replay
+        assert torch.equal(replayed._device_para, eager._device_para), replay
+        for se, sr in zip(eager.non_layerwise_step_contexts[0].optimizer_states, replayed.non_layerwise_step_contexts[0].optimizer_states):
+            assert torch.equal(se, sr), replay
+        assert not replayed._device_grad.any()
