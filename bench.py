@@ -29,6 +29,14 @@ N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 8
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
 # profiles/); None until measured for a workload.
 MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_657_000, "cfg3": 5_666_664_000, "cfg4": 23_958_221_000, "accumulate": 2_453_887_000}
+# The summary each literal is copied from; it carries the line "roofline.traffic = <bytes> B"
+# (tests/test_bench_contract.py checks that the two agree).
+TRAFFIC_SOURCE = {
+    "cfg2": "profiles/adam_tile_kernel_cfg2_llama7b_layer.md",
+    "cfg3": "profiles/grad_stats_and_adam_cfg3_overflow_path.md",
+    "cfg4": "profiles/adam_tile_kernel_cfg4_llama70b_layer.md",
+    "accumulate": "profiles/grad_accumulate_kernel_llama7b_layer.md",
+}
 
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
 
@@ -72,20 +80,31 @@ def _host_description():
     return {"cpu_model": model, "logical_cpus": os.cpu_count(), "numa_nodes": len(glob.glob("/sys/devices/system/node/node[0-9]*")) or 1}
 
 
+CPU_WARMUPS = 3
+
+
 def _time_cpu_adam(n, budget_s):
-    """1 warm-up call, then timed calls until the budget is used (at least 3, at most 20) of the
-    reference CPU Adam with fp32 gradients and an fp16 copy-out on n elements in host memory.
-    Returns (seconds per call as a 20-80 percentile mean, number of timed calls, kind, flavour)."""
+    """Warm-up calls until the time per call has settled, then timed calls until the budget is used (at least 3, at most 20)
+    of the reference CPU Adam with fp32 gradients and an fp16 copy-out on n elements in PINNED host
+    memory (where the reference keeps its optimizer state, flextrain/memory/__init__.py:255-277),
+    filled by the seeded generator. Returns (seconds per call as a 20-80 percentile mean, number of
+    timed calls, kind, flavour)."""
     import numpy as np
     import torch
 
     import oracle
+    from flextrain_amd import synth
+    from flextrain_amd.memory import pinned_empty
     ref = oracle.reference_module()
-    tp = torch.randn(n) * 0.02
-    tg = torch.randn(n) * 1e-3
-    tm = torch.zeros(n)
-    tv = torch.zeros(n)
-    th = torch.zeros(n, dtype=torch.float16)
+    tp, tg, tm, tv = (pinned_empty(n, torch.float32) for _ in range(4))
+    th = pinned_empty(n, torch.float16)
+    scratch = torch.empty(n, dtype=torch.float32, device="cuda")  # the generator's GPU side is the fast one
+    tp.copy_(synth.fill_(scratch, 0, 0, scale=0.02))
+    tg.copy_(synth.fill_(scratch, 0, 3, scale=1e-3))
+    del scratch
+    tm.zero_()
+    tv.zero_()
+    th.zero_()
     if ref is not None:
         kind, oid = "reference", 4242
         ref.create_adam(oid, HP["lr"], *HP["betas"], HP["eps"], HP["weight_decay"], True, False)
@@ -100,16 +119,24 @@ def _time_cpu_adam(n, budget_s):
         def call(t):
             oracle.adam_step(pn, gn, mn, vn, step=t, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
                              weight_decay=HP["weight_decay"], half_out=hn, half_dtype=oracle.F16)
-    call(1)
+    # Warm-up: at least CPU_WARMUPS calls, and on until three calls in a row agree within 5 % (the
+    # first second or so of a process's OpenMP work ran up to 40 % slower on the measured hosts:
+    # thread start-up, clock ramp, first use of the pinned pages), for 8 s at most.
+    warm, t_begin = [], time.perf_counter()
+    while len(warm) < CPU_WARMUPS or (min(warm[-3:]) < 0.95 * max(warm[-3:]) and time.perf_counter() - t_begin < 8.0) \
+            or time.perf_counter() - t_begin < 1.5:
+        t0 = time.perf_counter()
+        call(len(warm) + 1)
+        warm.append(time.perf_counter() - t0)
     times, t_begin = [], time.perf_counter()
     while len(times) < 20 and (len(times) < 3 or time.perf_counter() - t_begin < budget_s):
         t0 = time.perf_counter()
-        call(len(times) + 2)
+        call(len(times) + len(warm) + 1)
         times.append(time.perf_counter() - t0)
     if ref is not None:
         ref.destroy_adam(oid)
     flavour = getattr(ref, "flavour", f"libftoracle isa={oracle.best_isa()}")
-    return percentile_mean(times), len(times), kind, flavour
+    return percentile_mean(times), len(times), kind, flavour, len(warm)
 
 
 def cpu_baseline(n, budget_s=14.0):
@@ -120,38 +147,54 @@ def cpu_baseline(n, budget_s=14.0):
     the block size that probe itself uses (2**28 elements) and reported beside it."""
     import oracle
     threads = oracle.max_threads()
-    sec, calls, kind, flavour = _time_cpu_adam(n, budget_s)
+    sec, calls, kind, flavour, warmups = _time_cpu_adam(n, budget_s)
     out = {
         "value": n / sec, "unit": "elements/s", "cores": threads, "kind": kind,
-        "sample": f"{calls} timed calls (1 warm-up) of the CPU Adam with fp16 copy-out on {n} fp32 elements "
-                  f"in host memory, {threads} OpenMP threads, 20-80 percentile mean",
+        "sample": f"{calls} timed calls ({warmups} warm-ups) of the CPU Adam with fp16 copy-out on {n} fp32 elements "
+                  f"in pinned host memory, {threads} OpenMP threads, 20-80 percentile mean",
         "ms_per_call": sec * 1e3, "host_gbps": n * 30 / sec / 1e9, "flavour": flavour,
         "host": _host_description(),
     }
     block = 1 << 28
-    bsec, bcalls, _, _ = _time_cpu_adam(block, budget_s * 0.4)
+    bsec, bcalls, _, _, _ = _time_cpu_adam(block, budget_s * 0.4)
     out["reference_probe_block"] = {"elements": block, "value": block / bsec, "unit": "elements/s",
                                     "ms_per_call": bsec * 1e3, "timed_calls": bcalls}
     return out
 
 
-def bench_offload(args, torch, dev) -> int:
-    """cfg5: the full Llama-7B optimizer with fp32 master/m/v in pinned host DRAM, streamed through
-    the GPU in chunks (H2D -> fused AdamW -> D2H on three streams); bf16 gradients and the bf16
-    parameter copy stay on the GPU. One step = one pass over all elements, timed end to end."""
+def link_probe(torch):
+    """What the host link carries: the library's probe (two transfers in flight per direction; the
+    runtime's copies and a copy kernel; each direction alone and both at once) and the ceilings
+    derived from it. The unidirectional ceiling is the best figure any method reached in either
+    direction; two directions at once cannot carry more than twice that, so fractions of
+    ``full_duplex_ceiling_gbps`` cannot exceed 1."""
     import ctypes
 
-    from flextrain_amd import FlexTrainCPUAdam, _C
-    from flextrain_amd.memory import pinned_empty
+    from flextrain_amd import _C
+    r = _C.LinkProbe()
+    _C.check("ft_link_probe", _C.lib().ft_link_probe(1 << 30, 10, ctypes.byref(r)))
+    out = {name: getattr(r, name) for name, _ in _C.LinkProbe._fields_}
+    out["unidirectional_ceiling_gbps"] = max(r.h2d_copy, r.d2h_copy, r.h2d_kernel, r.d2h_kernel)
+    out["bidirectional_sum_measured_gbps"] = max(r.both_copy, r.both_kernel)
+    out["full_duplex_ceiling_gbps"] = 2 * out["unidirectional_ceiling_gbps"]
+    return out
 
+
+def measure_offload(args, torch, dev, layers, steps, warmup):
+    """cfg5: the Llama-7B optimizer with fp32 master/m/v in pinned host DRAM, streamed through the
+    GPU in chunks (H2D -> fused AdamW -> D2H on three streams); bf16 gradients and the bf16
+    parameter copy stay on the GPU. One step = one pass over all elements, timed end to end.
+    Returns (record, ok): the measurements and whether the streamed result equals the resident one."""
     import gc
+
+    from flextrain_amd import FlexTrainCPUAdam, _C, synth
+    from flextrain_amd.memory import pinned_empty
 
     n_full = 32 * N_7B_LAYER + 2 * 4096 * 32000
     chunk = args.chunk_elems
-    lib = _C.lib()
     # The whole state must be pinned (3 x 4 bytes per element). A machine that cannot pin that much
-    # runs the largest whole-layer prefix that fits, and the line says which fraction that is.
-    layers, p = args.layers, None
+    # runs the largest whole-layer prefix that fits, and the record says which fraction that is.
+    p = None
     while p is None:
         n = layers * N_7B_LAYER + 2 * 4096 * 32000
         t0 = time.perf_counter()
@@ -164,38 +207,34 @@ def bench_offload(args, torch, dev) -> int:
             gc.collect()
             layers -= 1
             if layers < 1:
-                print("cannot pin even one layer of optimizer state", file=sys.stderr)
-                return 1
+                raise RuntimeError("cannot pin even one layer of optimizer state")
     t_alloc = time.perf_counter() - t0
     g = torch.empty(n, dtype=torch.bfloat16, device=dev)
     h = torch.empty(n, dtype=torch.bfloat16, device=dev)
-    gen = torch.Generator(device=dev).manual_seed(0)
     t0 = time.perf_counter()
-    for lo in range(0, n, chunk):  # synthetic state is drawn on the GPU and copied down chunk by chunk
+    scratch = torch.empty(chunk, dtype=torch.float32, device=dev)
+    for lo in range(0, n, chunk):  # seeded state is generated on the GPU and copied down chunk by chunk
         hi = min(n, lo + chunk)
         k = hi - lo
-        p[lo:hi].copy_(torch.randn(k, device=dev, generator=gen) * 0.02)
-        m[lo:hi].copy_(torch.randn(k, device=dev, generator=gen) * 1e-4)
-        v[lo:hi].copy_(torch.rand(k, device=dev, generator=gen) * 1e-6)
-        g[lo:hi] = (torch.randn(k, device=dev, generator=gen) * 1e-3).to(torch.bfloat16)
+        p[lo:hi].copy_(synth.fill_(scratch[:k], 0, 0, scale=0.02, first_index=lo))
+        m[lo:hi].copy_(synth.fill_(scratch[:k], 0, 1, scale=1e-4, first_index=lo))
+        v[lo:hi].copy_(synth.fill_(scratch[:k], 0, 2, kind=synth.UNIFORM, scale=1e-6, first_index=lo))
+    synth.fill_(g, 0, 3, scale=1e-3)
     torch.cuda.synchronize()
+    del scratch
     t_init = time.perf_counter() - t0
 
-    link = {}
-    out = ctypes.c_double()
-    for name, direction in (("h2d", 0), ("d2h", 1), ("both", 2)):
-        _C.check("ft_link_bandwidth", lib.ft_link_bandwidth(1 << 30, 20, direction, ctypes.byref(out)))
-        link[name] = out.value
+    link = link_probe(torch)
 
     eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=args.slots, **HP)
-    # keep copies of two chunks to check the streamed result against the resident kernel afterwards
-    probes = [0, (n // chunk // 2) * chunk, ((n - 1) // chunk) * chunk]
+    # keep copies of three chunks to check the streamed result against the resident kernel afterwards
+    probes = sorted({0, (n // chunk // 2) * chunk, ((n - 1) // chunk) * chunk})
     before = {lo: tuple(t[lo:min(n, lo + chunk)].to(dev) for t in (p, m, v)) for lo in probes}
     group = {"step": 100}
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         eng._step(group, h, p, g, m, v)
     walls, devs = [], []
-    for _ in range(args.steps):
+    for _ in range(steps):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         eng._step(group, h, p, g, m, v)  # blocks until the host arrays hold the new values
@@ -208,34 +247,48 @@ def bench_offload(args, torch, dev) -> int:
     for lo, (bp, bm, bv) in before.items():
         hi = min(n, lo + chunk)
         bh = torch.empty(hi - lo, dtype=torch.bfloat16, device=dev)
-        for _ in range(args.warmup + args.steps):
+        for _ in range(warmup + steps):
             res._step(group, bh, bp, g[lo:hi], bm, bv)
         torch.cuda.synchronize()
         ok = ok and torch.equal(bp.cpu(), p[lo:hi]) and torch.equal(bm.cpu(), m[lo:hi]) and torch.equal(bv.cpu(), v[lo:hi]) \
             and torch.equal(bh, h[lo:hi])
     sec = sum(walls) / len(walls)
     one_way = n * 12 / sec / 1e9
-    out_json = {
-        "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
-        "value": n / sec, "unit": "elements/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": sec * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": f"cfg5: offloaded Llama-7B optimizer ({layers} of 32 layers + embedding + lm_head), "
-                               "fp32 p/m/v in pinned host DRAM streamed in chunks, bf16 grads and copy on GPU",
-                   "elements": n, "fraction_of_full_7b": n / n_full, "chunk_elems": chunk, "slots": args.slots,
-                   "chunks": -(-n // chunk)},
-        "link": {
-            "measured_h2d_gbps": link["h2d"], "measured_d2h_gbps": link["d2h"], "measured_bidirectional_gbps": link["both"],
-            "achieved_each_way_gbps": one_way, "achieved_total_gbps": 2 * one_way,
-            "frac_of_unidirectional": one_way / min(link["h2d"], link["d2h"]),
-            "frac_of_bidirectional": 2 * one_way / link["both"],
-            "bytes_each_way": n * 12, "device_time_ms": sum(devs) / len(devs) * 1e3,
-        },
-        "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_tile_kernel per chunk",
-                     "achieved": 2 * one_way, "peak": link["both"], "unit": "GB/s", "frac": 2 * one_way / link["both"],
-                     "traffic": None},
+    record = {
+        "workload": f"cfg5: offloaded Llama-7B optimizer ({layers} of 32 layers + embedding + lm_head), "
+                    "fp32 p/m/v in pinned host DRAM streamed in chunks, bf16 grads and copy on GPU",
+        "elements": n, "fraction_of_full_7b": n / n_full, "chunk_elems": chunk, "slots": args.slots, "chunks": -(-n // chunk),
+        "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "elements_per_s": n / sec,
+        "bytes_each_way": n * 12, "achieved_each_way_gbps": one_way, "achieved_total_gbps": 2 * one_way,
+        "device_time_ms": sum(devs) / len(devs) * 1e3,
+        "link": link,
+        "frac_of_unidirectional": one_way / link["unidirectional_ceiling_gbps"],
+        "frac_of_bidirectional_measured": 2 * one_way / link["bidirectional_sum_measured_gbps"],
         "setup": {"pinned_alloc_s": t_alloc, "init_s": t_init, "pinned_gb": 3 * n * 4 / 1e9},
         "streamed_equals_resident_on_probe_chunks": bool(ok),
+    }
+    del p, m, v, g, h, before
+    gc.collect()
+    torch.cuda.empty_cache()
+    return record, ok
+
+
+def bench_offload(args, torch, dev) -> int:
+    rec, ok = measure_offload(args, torch, dev, args.layers, args.steps, args.warmup)
+    link = rec["link"]
+    out_json = {
+        "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
+        "value": rec["elements_per_s"], "unit": "elements/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": rec["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {k: rec[k] for k in ("workload", "elements", "fraction_of_full_7b", "chunk_elems", "slots", "chunks")},
+        "offload": rec,
+        # Both directions at the unidirectional ceiling is the most a full-duplex link can carry: a
+        # fraction of it cannot exceed 1 (what both directions reach when probed together is lower
+        # and is listed beside it).
+        "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_tile_kernel per chunk",
+                     "achieved": rec["achieved_total_gbps"], "peak": link["full_duplex_ceiling_gbps"], "unit": "GB/s",
+                     "frac": rec["achieved_total_gbps"] / link["full_duplex_ceiling_gbps"], "traffic": None},
     }
     print(json.dumps(out_json), flush=True)
     return 0 if ok else 3
@@ -292,7 +345,7 @@ def bench_accumulate(args, torch, dev) -> int:
                                "statistics of the result in the same pass", "elements": n},
         "roofline": {"bound": "hbm", "kernel": "grad_accumulate_kernel", "achieved": main["achieved_gbps"],
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": main["achieved_gbps"] / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES["accumulate"],
+                     "traffic": MEASURED_TRAFFIC_BYTES["accumulate"], "traffic_source": TRAFFIC_SOURCE["accumulate"],
                      "algorithmic_bytes_per_launch": n * 12, "kernel_ms_avg": main["ms_avg"]},
         "variants": results,
     }), flush=True)
@@ -342,11 +395,7 @@ def bench_pipeline(args, torch, dev) -> int:
                 return 1
     grads = (torch.randn(n, device=dev) * 1e-3).to(torch.bfloat16)
     share = n // mb
-    link = {}
-    out = ctypes.c_double()
-    for name, direction in (("h2d", 0), ("d2h", 1), ("both", 2)):
-        _C.check("ft_link_bandwidth", lib.ft_link_bandwidth(1 << 30, 10, direction, ctypes.byref(out)))
-        link[name] = out.value
+    link = link_probe(torch)
 
     def iteration():
         opt.update_states()
@@ -378,13 +427,12 @@ def bench_pipeline(args, torch, dev) -> int:
                                "fp32 state in pinned host DRAM, bf16 grads and parameters on GPU",
                    "elements": total, "units": units, "micro_batches": mb, "chunk_elems": args.chunk_elems,
                    "slots": args.slots, "unit_windows": args.windows},
-        "link": {"measured_h2d_gbps": link["h2d"], "measured_d2h_gbps": link["d2h"],
-                 "measured_bidirectional_gbps": link["both"], "achieved_each_way_gbps": one_way,
-                 "achieved_total_gbps": 2 * one_way, "frac_of_unidirectional": one_way / min(link["h2d"], link["d2h"]),
-                 "frac_of_bidirectional": 2 * one_way / link["both"]},
+        "link": dict(link, achieved_each_way_gbps=one_way, achieved_total_gbps=2 * one_way,
+                     frac_of_unidirectional=one_way / link["unidirectional_ceiling_gbps"],
+                     frac_of_bidirectional_measured=2 * one_way / link["bidirectional_sum_measured_gbps"]),
         "roofline": {"bound": "host-link", "kernel": "hipMemcpyAsync H2D/D2H + adam_tile_kernel per share",
-                     "achieved": 2 * one_way, "peak": link["both"], "unit": "GB/s", "frac": 2 * one_way / link["both"],
-                     "traffic": None},
+                     "achieved": 2 * one_way, "peak": link["full_duplex_ceiling_gbps"], "unit": "GB/s",
+                     "frac": 2 * one_way / link["full_duplex_ceiling_gbps"], "traffic": None},
     }), flush=True)
     return 0
 
@@ -578,6 +626,8 @@ def main() -> int:
     ap.add_argument("--resident", action="store_true",
                     help="pipeline: keep the fp32 state of every unit in HBM instead of pinned host memory")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-offload-record", action="store_true",
+                    help="cfg2: leave out the offloaded-streaming sub-record (cfg5 on the largest pinnable prefix, about 12 s)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="before the timed region, run 3 plain device copies of one fp32 array of the workload "
                          "(known size: 4 bytes/element read + 4 written) so that a rocprofv3 --pmc run of this "
@@ -698,6 +748,7 @@ def main() -> int:
         "roofline": {
             "bound": "hbm", "kernel": "adam_tile_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic_source": TRAFFIC_SOURCE.get(args.workload),
             "algorithmic_bytes_per_launch": alg_bytes, "kernel_ms_avg": upd_avg, "kernel_ms_min": min(upd_ms),
             "kernel_ms_p20_80": percentile_mean(upd_ms),
         },
@@ -706,9 +757,18 @@ def main() -> int:
         pre_avg = sum(pre_ms) / len(pre_ms)
         out["stats_pass"] = {"kernel": "grad_stats_kernel", "ms_avg": pre_avg, "bytes": n * 2,
                              "achieved_gbps": n * 2 / (pre_avg * 1e-3) / 1e9}
+    del p, g, m, v, h
+    torch.cuda.empty_cache()
+    if args.workload == "cfg2" and not args.no_offload_record:
+        # The path's second target rides along: the offloaded optimizer streamed over the host link
+        # (cfg5 at the largest size this machine pins), 1 warm-up + 3 steps, beside the link probe.
+        try:
+            out["offload"], ok = measure_offload(args, torch, dev, args.layers, steps=3, warmup=1)
+            if not ok:
+                out["offload"]["error"] = "streamed and resident results differ on the probe chunks"
+        except Exception as exc:  # the headline figure must not depend on how much this machine can pin
+            out["offload"] = {"error": f"{type(exc).__name__}: {exc}"}
     if not args.no_cpu_baseline:
-        del p, g, m, v, h
-        torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline(min(n, N_7B_LAYER))
     print(json.dumps(out), flush=True)
     return 0

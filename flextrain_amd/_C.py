@@ -28,6 +28,12 @@ class AdamSegment(ctypes.Structure):
     ]
 
 
+class LinkProbe(ctypes.Structure):
+    """Mirror of ``ft_link_probe_t`` (GB/s; ``both_*`` is the sum of the two directions)."""
+
+    _fields_ = [(name, c_double) for name in ("h2d_copy", "d2h_copy", "both_copy", "h2d_kernel", "d2h_kernel", "both_kernel")]
+
+
 EXPORTS = {
     # name: (restype, argtypes)
     "ft_last_error": (c_char_p, []),
@@ -60,6 +66,7 @@ EXPORTS = {
     "ft_offload_stream_wait": (c_int, [c_void_p, c_void_p, c_int]),
     "ft_offload_wait": (c_int, [c_void_p]),
     "ft_offload_elapsed_ms": (c_int, [c_void_p, POINTER(c_float)]),
+    "ft_link_probe": (c_int, [c_size_t, c_int, POINTER(LinkProbe)]),
     "ft_link_bandwidth": (c_int, [c_size_t, c_int, c_int, POINTER(c_double)]),
     "ft_synth_fill": (c_int, [c_void_p, c_int, c_size_t, c_uint64, c_uint32, c_uint64, c_int, c_float, c_void_p]),
     "ft_synth_fill_host": (c_int, [c_void_p, c_int, c_size_t, c_uint64, c_uint32, c_uint64, c_int, c_float]),

@@ -231,10 +231,19 @@ int ft_offload_stream_wait(void* handle, void* stream, int what);
 int ft_offload_wait(void* handle);
 int ft_offload_elapsed_ms(void* handle, float* out_ms);
 
-/* Host-link probe used to put the offloaded step next to what the link can do: copies `bytes`
- * between pinned host and device memory `iters` times and reports GB/s (1e9 bytes/s).
- * direction: 0 = host-to-device, 1 = device-to-host, 2 = both at once (sum of both reported).
- * The method follows the reference's own probe (flextrain/auto_config.py:184-215). */
+/* Host-link probe used to put the offloaded step next to what the link can do. The method follows
+ * the reference's own probe (flextrain/auto_config.py:184-215: timed copies between pinned host and
+ * device memory), hardened into a ceiling: `bytes` are moved per direction and iteration, every
+ * figure the better of one and of two transfers in flight, once with the runtime's copies (*_copy) and once with a copy
+ * kernel that reads or writes the pinned memory itself (*_kernel), host-to-device alone,
+ * device-to-host alone, and both at once (both_*: the SUM of the two directions). GB/s = 1e9 bytes/s.
+ * ft_link_bandwidth returns the better of the two methods for one direction code
+ * (0 = host-to-device, 1 = device-to-host, 2 = both at once, summed). */
+typedef struct ft_link_probe_t {
+    double h2d_copy, d2h_copy, both_copy;
+    double h2d_kernel, d2h_kernel, both_kernel;
+} ft_link_probe_t;
+int ft_link_probe(size_t bytes, int iters, ft_link_probe_t* out);
 int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps);
 
 /* ---- synthetic inputs ----------------------------------------------------------------------
