@@ -37,3 +37,21 @@ def cuda():
     if not torch.cuda.is_available():
         pytest.skip("no GPU in this environment")
     return torch.device("cuda", 0)
+
+
+# Facts a passing test wants on record (how much of a configuration a machine could hold, say):
+# `pytest -q` drops the output of passing tests, the terminal summary stays.
+_SUMMARY_LINES = []
+
+
+@pytest.fixture
+def summary_line():
+    """Callable that puts one line into the run's terminal summary."""
+    return _SUMMARY_LINES.append
+
+
+def pytest_terminal_summary(terminalreporter):
+    if _SUMMARY_LINES:
+        terminalreporter.section("coverage notes")
+        for line in _SUMMARY_LINES:
+            terminalreporter.write_line(line)

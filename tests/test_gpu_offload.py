@@ -423,16 +423,26 @@ def test_engine_grows_its_chunk_for_long_steps(cuda, oracle, mode):
         _assert_equal_bits(f"grown chunk mode={mode} n={n}", p, m, v, h, want, torch.bfloat16)
 
 
-def test_config5_offloaded_7b_optimizer(cuda, oracle):
-    """The offloaded Llama-7B optimizer at the largest size this machine can pin (all 32 layers +
-    embedding + lm_head = 6.74e9 elements need 81 GB of pinned memory; a machine that refuses that
-    much runs the largest whole-layer prefix): 64 Mi-element chunks, one AdamW step at t = 100.
-    Checked by (1) the oracle on three whole chunks (first, middle, last ragged one) and
-    (2) bit-equality with the resident kernel on every chunk."""
+CFG5_MIN_LAYERS = 24  # a machine that cannot pin even this much of the 32-layer optimizer fails the test
+
+
+def test_config5_offloaded_7b_optimizer(cuda, oracle, summary_line):
+    """The offloaded Llama-7B optimizer: 32 layers + embedding + lm_head = 6,738,411,520 elements,
+    81 GB of pinned fp32 state, 101 chunks of 64 Mi elements, one AdamW step at t = 100. A machine
+    that refuses to pin that much in one piece (the measured ones stop near 64 GiB) covers it in two
+    passes over the largest slab it can pin: pass 1 streams the elements from 0 up, pass 2 the
+    elements up to the end of the optimizer starting at a chunk boundary, so that every chunk 0..100
+    is streamed with its true extent and its true element indices (the inputs are a function of the
+    element index). Fewer than 24 layers' worth of slab is a failure, not a smaller test.
+    Each pass is checked by (1) the oracle on three whole chunks (first, middle, last) and (2)
+    bit-equality with the resident kernel on every chunk. The reached size goes into the summary."""
     import gc
-    from flextrain_amd import FlexTrainCPUAdam, _C
+    from flextrain_amd import FlexTrainCPUAdam, _C, synth
     from flextrain_amd.memory import pinned_empty
     layer, chunk = 202_383_360, 64 * 1024 * 1024
+    n_full = 32 * layer + 2 * 4096 * 32000
+    total_chunks = -(-n_full // chunk)
+    assert total_chunks == 101
     layers, state = 32, None
     while state is None:
         n = layers * layer + 2 * 4096 * 32000
@@ -444,43 +454,59 @@ def test_config5_offloaded_7b_optimizer(cuda, oracle):
             state = None
             gc.collect()
             layers -= 1
-            assert layers >= 1
-    p, m, v = state
-    print(f"[cfg5] pinned {3 * n * 4 / 1e9:.1f} GB: {layers} of 32 layers, {n} elements, {-(-n // chunk)} chunks", flush=True)
-    g = torch.empty(n, dtype=torch.bfloat16, device=cuda)
-    h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
-    gen = torch.Generator(device=cuda).manual_seed(0)
-    for lo in range(0, n, chunk):
-        hi = min(n, lo + chunk)
-        p[lo:hi].copy_(torch.randn(hi - lo, device=cuda, generator=gen) * 0.02)
-        m[lo:hi].copy_(torch.randn(hi - lo, device=cuda, generator=gen) * 1e-4)
-        v[lo:hi].copy_(torch.rand(hi - lo, device=cuda, generator=gen) * 1e-6)
-        g[lo:hi] = (torch.randn(hi - lo, device=cuda, generator=gen) * 1e-3).to(torch.bfloat16)
-    torch.cuda.synchronize()
-    nchunks = -(-n // chunk)
-    probes = sorted({0, nchunks // 2, nchunks - 1})
-    want = {}
-    for c in probes:
-        lo, hi = c * chunk, min(n, (c + 1) * chunk)
-        want[c] = _oracle(oracle, p[lo:hi], g[lo:hi], m[lo:hi], v[lo:hi], 100, torch.bfloat16)
-    # resident results for every chunk, kept as 64-bit checksums of the raw bits
+            assert layers >= CFG5_MIN_LAYERS, f"this machine cannot pin {CFG5_MIN_LAYERS} layers of optimizer state"
+    P, M, V = state
+    G = torch.empty(n, dtype=torch.bfloat16, device=cuda)
+    H = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    scratch = torch.empty(chunk, dtype=torch.float32, device=cuda)
     res = FlexTrainCPUAdam(**HP)
-    sums = []
-    for lo in range(0, n, chunk):
-        hi = min(n, lo + chunk)
-        dp, dm, dv = p[lo:hi].to(cuda), m[lo:hi].to(cuda), v[lo:hi].to(cuda)
-        dh = torch.empty(hi - lo, dtype=torch.bfloat16, device=cuda)
-        res._step({"step": 100}, dh, dp, g[lo:hi], dm, dv)
-        sums.append(tuple(int(t.view(torch.int32).to(torch.int64).sum().item()) for t in (dp, dm, dv)) +
-                    (int(dh.view(torch.int16).to(torch.int64).sum().item()),))
     eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=3, **HP)
-    eng._step({"step": 100}, h, p, g, m, v)
-    print(f"[cfg5] streamed step: {eng.last_offload_ms():.1f} ms, {n * 12 / eng.last_offload_ms() / 1e6:.1f} GB/s each way", flush=True)
-    for c in probes:
-        lo, hi = c * chunk, min(n, (c + 1) * chunk)
-        _assert_equal_bits(f"cfg5 chunk {c}", p[lo:hi], m[lo:hi], v[lo:hi], h[lo:hi], want[c], torch.bfloat16)
-    for i, lo in enumerate(range(0, n, chunk)):
-        hi = min(n, lo + chunk)
-        got = tuple(int(t[lo:hi].to(cuda).view(torch.int32).to(torch.int64).sum().item()) for t in (p, m, v)) + \
-            (int(h[lo:hi].view(torch.int16).to(torch.int64).sum().item()),)
-        assert got == sums[i], f"chunk {i}: streamed and resident results differ"
+
+    # pass 1: elements [0, n); pass 2: [first2, n_full), first2 the first chunk boundary that fits
+    first2 = -(-(n_full - n) // chunk) * chunk if n < n_full else n_full
+    passes = [(0, n)] + ([(first2, n_full - first2)] if first2 < n_full else [])
+    seen_chunks = set()
+    for number, (first, count) in enumerate(passes, 1):
+        p, m, v, g, h = P[:count], M[:count], V[:count], G[:count], H[:count]
+        for lo in range(0, count, chunk):  # element i of the optimizer is a function of i alone
+            hi = min(count, lo + chunk)
+            k = hi - lo
+            p[lo:hi].copy_(synth.fill_(scratch[:k], 0, 0, scale=0.02, first_index=first + lo))
+            m[lo:hi].copy_(synth.fill_(scratch[:k], 0, 1, scale=1e-4, first_index=first + lo))
+            v[lo:hi].copy_(synth.fill_(scratch[:k], 0, 2, kind=synth.UNIFORM, scale=1e-6, first_index=first + lo))
+        synth.fill_(g, 0, 3, scale=1e-3, first_index=first)
+        h.zero_()
+        torch.cuda.synchronize()
+        nchunks = -(-count // chunk)
+        probes = sorted({0, nchunks // 2, nchunks - 1})
+        want = {}
+        for c in probes:
+            lo, hi = c * chunk, min(count, (c + 1) * chunk)
+            want[c] = _oracle(oracle, p[lo:hi], g[lo:hi], m[lo:hi], v[lo:hi], 100, torch.bfloat16)
+        # resident results for every chunk, kept as 64-bit checksums of the raw bits
+        sums = []
+        for lo in range(0, count, chunk):
+            hi = min(count, lo + chunk)
+            dp, dm, dv = p[lo:hi].to(cuda), m[lo:hi].to(cuda), v[lo:hi].to(cuda)
+            dh = torch.empty(hi - lo, dtype=torch.bfloat16, device=cuda)
+            res._step({"step": 100}, dh, dp, g[lo:hi], dm, dv)
+            sums.append(tuple(int(t.view(torch.int32).to(torch.int64).sum().item()) for t in (dp, dm, dv)) +
+                        (int(dh.view(torch.int16).to(torch.int64).sum().item()),))
+        eng._step({"step": 100}, h, p, g, m, v)
+        rate = count * 12 / eng.last_offload_ms() / 1e6
+        print(f"[cfg5 pass {number}] elements [{first}, {first + count}): {eng.last_offload_ms():.1f} ms, {rate:.1f} GB/s each way", flush=True)
+        for c in probes:
+            lo, hi = c * chunk, min(count, (c + 1) * chunk)
+            _assert_equal_bits(f"cfg5 pass {number} chunk {first // chunk + c}", p[lo:hi], m[lo:hi], v[lo:hi], h[lo:hi], want[c], torch.bfloat16)
+        for i, lo in enumerate(range(0, count, chunk)):
+            hi = min(count, lo + chunk)
+            got = tuple(int(t[lo:hi].to(cuda).view(torch.int32).to(torch.int64).sum().item()) for t in (p, m, v)) + \
+                (int(h[lo:hi].view(torch.int16).to(torch.int64).sum().item()),)
+            assert got == sums[i], f"pass {number} chunk {i}: streamed and resident results differ"
+            if first % chunk == 0 and (hi - lo == chunk or first + hi == n_full):
+                seen_chunks.add(first // chunk + i)  # streamed with its true extent
+        summary_line(f"cfg5 pass {number}: streamed elements [{first:,}, {first + count:,}) of {n_full:,} "
+                     f"({3 * count * 4 / 1e9:.1f} GB pinned state, {nchunks} chunks) at {rate:.1f} GB/s each way")
+    assert seen_chunks == set(range(total_chunks)), sorted(set(range(total_chunks)) - seen_chunks)
+    summary_line(f"cfg5: {layers} of 32 layers fit one pinned slab; all {total_chunks} chunks of the full optimizer streamed "
+                 f"in {len(passes)} pass(es)")
