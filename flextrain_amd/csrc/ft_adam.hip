@@ -11,6 +11,7 @@
 
 #include <atomic>
 #include <cmath>
+#include <map>
 #include <mutex>
 #include <unordered_map>
 
@@ -41,8 +42,12 @@ thread_local std::string t_last_error;
 std::mutex g_mu;
 std::unordered_map<int, fth::AdamObject> g_adams;
 std::unordered_map<int, int> g_cu_count;      // device -> compute units
-std::unordered_map<int, void*> g_stats_ws;    // device -> library-owned statistics scratch
-std::unordered_map<int, size_t> g_stats_ws_bytes;
+struct OwnedScratch {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+// (device, stream) -> library-owned statistics scratch: calls on different streams never share one
+std::map<std::pair<int, hipStream_t>, OwnedScratch> g_stats_ws;
 int g_adam_waves_per_cu = FT_ADAM_WAVES_PER_CU;
 std::unordered_map<int, int> g_lds_per_cu;   // device -> bytes of LDS per compute unit
 std::atomic<int> g_stats_blocks_per_cu{FT_STATS_BLOCKS_PER_CU};  // read without the lock
@@ -324,10 +329,11 @@ extern "C" size_t ft_grad_stats_workspace_bytes(void);
 
 namespace {
 
-// The caller's scratch if given (checked against `need` bytes), else the per-device buffer the
-// library owns, grown when a call needs more than it holds (hipFree waits for the device, so work
-// still using the old buffer has finished before it goes away).
-int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need, ftk::StatsPartial** out)
+// The caller's scratch if given (checked against `need` bytes), else a buffer the library owns for
+// this (device, stream), grown when a call needs more than it holds (hipFree waits for the device,
+// so work still using the old buffer has finished before it goes away). Calls on one stream are
+// ordered, so they may share a buffer; calls on different streams get different ones.
+int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need, hipStream_t stream, ftk::StatsPartial** out)
 {
     ftk::StatsPartial* parts = static_cast<ftk::StatsPartial*>(workspace);
     if (parts) {
@@ -339,17 +345,21 @@ int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need
         int dev = 0;
         FT_HIP(hipGetDevice(&dev));
         std::lock_guard<std::mutex> lk(g_mu);
-        auto it = g_stats_ws.find(dev);
-        if (it == g_stats_ws.end() || g_stats_ws_bytes[dev] < need) {
-            if (it != g_stats_ws.end()) FT_HIP(hipFree(it->second));
+        OwnedScratch& own = g_stats_ws[std::make_pair(dev, stream)];
+        if (own.bytes < need) {
+            if (own.ptr) FT_HIP(hipFree(own.ptr));
+            own.ptr = nullptr;
+            own.bytes = 0;
             void* w = nullptr;
-            FT_HIP(hipMalloc(&w, need));
-            g_stats_ws[dev] = w;
-            g_stats_ws_bytes[dev] = need;
-            parts = static_cast<ftk::StatsPartial*>(w);
-        } else {
-            parts = static_cast<ftk::StatsPartial*>(it->second);
+            hipError_t e = hipMalloc(&w, need);
+            if (e != hipSuccess) {
+                (void)hipGetLastError();
+                return fth::fail(FT_ENOMEM, "hipMalloc(%zu) for the statistics scratch failed: %s", need, hipGetErrorString(e));
+            }
+            own.ptr = w;
+            own.bytes = need;
         }
+        parts = static_cast<ftk::StatsPartial*>(own.ptr);
     }
     *out = parts;
     return FT_OK;
@@ -611,7 +621,7 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
     if (n > 0 && !aligned(g, elem_size(g_dtype))) return fth::fail(FT_EALIGN, "g is not aligned to its element size");
 
     ftk::StatsPartial* parts = nullptr;
-    int wrc = resolve_stats_workspace(workspace, workspace_bytes, ft_grad_stats_workspace_bytes(), &parts);
+    int wrc = resolve_stats_workspace(workspace, workspace_bytes, ft_grad_stats_workspace_bytes(), stream, &parts);
     if (wrc != FT_OK) return wrc;
 
     const size_t esz = elem_size(g_dtype);
@@ -700,7 +710,7 @@ int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t 
         if (wrc != FT_OK) return wrc;
         parts = static_cast<ftk::StatsPartial*>(ptr);
     } else if (stats) {
-        int wrc = resolve_stats_workspace(workspace, workspace_bytes, accumulate_workspace_bytes(n), &parts);
+        int wrc = resolve_stats_workspace(workspace, workspace_bytes, accumulate_workspace_bytes(n), stream, &parts);
         if (wrc != FT_OK) return wrc;
     }
     ft_grad_stats_t* out = static_cast<ft_grad_stats_t*>(stats_out);

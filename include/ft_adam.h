@@ -121,8 +121,10 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
  * ft_grad_stats: one pass over g; writes (accumulate == 0) or adds (accumulate != 0) the count
  * of inf/nan elements and the sum of squares of (float)g * pre_mult into *out (device).
  * workspace: device scratch of at least ft_grad_stats_workspace_bytes() bytes, or NULL to use a
- * per-device buffer the library allocates on first use (calls that share it must be ordered on
- * one stream).
+ * buffer the library keeps per (device, stream): it is allocated on first use and re-allocated when
+ * a call needs a larger one (so a NULL-workspace call may allocate and wait for the device; bring
+ * a workspace, or use ft_grad_accumulate_static, where that is not acceptable). Calls on different
+ * streams never share a library-owned buffer.
  */
 size_t ft_grad_stats_workspace_bytes(void);
 int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate,

@@ -253,3 +253,38 @@ def test_step_keywords_check_overflow_and_clip(cuda, oracle):
 
     with pytest.raises(ValueError):
         eng.step(ctxs, check_overflow=True, grad_mult=0.5)
+
+
+def test_library_owned_scratch_is_per_stream(cuda, oracle):
+    """ft_grad_stats and ft_grad_accumulate without a workspace (the library keeps one per device
+    and stream): calls interleaved on two streams over different gradients, growing the scratch in
+    between, must each report their own statistics."""
+    from flextrain_amd import _C
+    lib = _C.lib()
+    streams = [torch.cuda.Stream(device=cuda) for _ in range(2)]
+    sizes = [(3_000_001, 2_000_000), (5_000_003, 700_001)]
+    gen = torch.Generator(device=cuda).manual_seed(21)
+    grads = [[(torch.randn(n, device=cuda, generator=gen) * (k + 1)).to(torch.bfloat16) for n in sizes[k]] for k in range(2)]
+    accs = [[torch.zeros(n, device=cuda) for n in sizes[k]] for k in range(2)]
+    grads[1][0][12] = float("inf")
+    records = [[torch.zeros(2, dtype=torch.float64, device=cuda) for _ in range(3)] for _ in range(2)]
+    torch.cuda.synchronize()
+    for round_ in range(2):
+        for k, stream in enumerate(streams):
+            g = grads[k][round_]
+            _C.check("ft_grad_stats", lib.ft_grad_stats(g.data_ptr(), _C.BF16, g.numel(), 0.5, records[k][round_].data_ptr(), 0,
+                                                        None, 0, stream.cuda_stream))
+    for k, stream in enumerate(streams):  # the accumulation pass needs a larger scratch: the buffers grow
+        g, acc = grads[k][0], accs[k][0]
+        _C.check("ft_grad_accumulate", lib.ft_grad_accumulate(acc.data_ptr(), _C.F32, g.data_ptr(), _C.BF16, g.numel(), 1.0, 0, 0.5,
+                                                              records[k][2].data_ptr(), 0, None, 0, stream.cuda_stream))
+    torch.cuda.synchronize()
+    for k in range(2):
+        for round_ in range(2):
+            bad, sumsq = oracle.grad_stats(_bits(grads[k][round_]), CODE[torch.bfloat16], pre_mult=0.5)
+            got = records[k][round_].cpu()
+            assert int(got[0:1].view(torch.int64).item()) == bad == (1 if (k, round_) == (1, 0) else 0)
+            assert abs(float(got[1]) - sumsq) <= 2 * NORM_RTOL * sumsq
+        bad, sumsq = oracle.grad_stats(_bits(grads[k][0]), CODE[torch.bfloat16], pre_mult=0.5)
+        got = records[k][2].cpu()  # acc was zero: the accumulated values are the gradients, widened
+        assert int(got[0:1].view(torch.int64).item()) == bad and abs(float(got[1]) - sumsq) <= 2 * NORM_RTOL * sumsq
