@@ -684,8 +684,7 @@ def main() -> int:
     def one_step():
         if guard is not None:
             guard.begin()
-            guard.add(g, loss_scale=scale)
-            ctl = guard.decide_async(loss_scale=scale, max_grad_norm=max_norm)
+            ctl = guard.add_and_decide(g, loss_scale=scale, max_grad_norm=max_norm)
             eng._step(group, h, p, g, m, v, control=ctl)
         else:
             eng._step(group, h, p, g, m, v)
@@ -711,8 +710,7 @@ def main() -> int:
         if guard is not None:
             ev[i][0].record()
             guard.begin()
-            guard.add(g, loss_scale=scale)
-            ctl = guard.decide_async(loss_scale=scale, max_grad_norm=max_norm)
+            ctl = guard.add_and_decide(g, loss_scale=scale, max_grad_norm=max_norm)
             ev[i][1].record()
             eng._step(group, h, p, g, m, v, control=ctl)
         else:  # no statistics pass: one event pair around the update is all there is to time

@@ -50,6 +50,10 @@ EXPORTS = {
     "ft_grad_accumulate_workspace_bytes": (c_size_t, [c_size_t]),
     "ft_grad_accumulate": (c_int, [c_void_p, c_int, c_void_p, c_int, c_size_t, c_float, c_int, c_float, c_void_p, c_int,
                                    c_void_p, c_size_t, c_void_p]),
+    "ft_grad_decide": (c_int, [c_void_p, c_int, c_size_t, c_float, c_void_p, c_int, c_float, c_float, c_void_p, c_void_p, c_size_t,
+                               c_void_p]),
+    "ft_grad_accumulate_decide": (c_int, [c_void_p, c_int, c_void_p, c_int, c_size_t, c_float, c_int, c_float, c_void_p, c_int,
+                                          c_float, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ft_grad_accumulate_static": (c_int, [c_void_p, c_int, c_void_p, c_int, c_size_t, c_float, c_int, c_float, c_void_p, c_int,
                                           c_void_p]),
     "ft_grad_control": (c_int, [c_void_p, c_float, c_float, c_void_p, c_void_p]),

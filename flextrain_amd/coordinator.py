@@ -331,8 +331,11 @@ class FlexTrainOptsCoordinator:
         iteration (its own gradients and those of the units that finished before it)."""
         if not self._guarded or self._defer:
             return
-        self._gather_unit_statistics(self._gpu_bwd_step_grads)
-        self._iter_guard.decide_async(loss_scale=self.loss_scale, out=self._unit_controls[unit_index])
+        if self._gradacc_dtype_incompatible:  # the fused accumulation pass has gathered the unit's statistics
+            self._iter_guard.decide_async(loss_scale=self.loss_scale, out=self._unit_controls[unit_index])
+        else:
+            self._iter_guard.add_and_decide(self._gpu_bwd_step_grads, loss_scale=self.loss_scale,
+                                            out=self._unit_controls[unit_index])
 
     def _finish_iteration_statistics(self):
         """Reads the iteration's record back (one small copy), drives the loss scaler and returns the

@@ -367,6 +367,13 @@ int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need
 
 constexpr int kReduceBlocks = 256;  // second-level blocks of the accumulation pass's statistics
 
+// A decision to take in the last launch of a statistics pass (ctl == nullptr: none).
+struct Decide {
+    float inv_scale = 1.0f;
+    float max_norm = 0.0f;
+    ft_step_control_t* ctl = nullptr;
+};
+
 // Statistics scratch of ft_grad_accumulate_static: block partials followed by one wavefront partial
 // per 256 elements, for calls of up to FT_STATIC_MAX_ELEMS elements. It is part of the loaded code
 // object, so every GPU the library runs on holds its own copy (8.1 MiB) until the process ends.
@@ -403,7 +410,7 @@ size_t accumulate_workspace_bytes(size_t n)
 
 template <int AT, int GT, bool ZERO, bool STATS>
 int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, float scale, float pre_mult,
-                      ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, hipStream_t stream)
+                      ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, const Decide& dec, hipStream_t stream)
 {
     constexpr size_t asz = (AT == FT_F32) ? 4 : 2, gsz = (GT == FT_F32) ? 4 : 2;
     int reduce_blocks = 0;
@@ -435,7 +442,7 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
         hipLaunchKernelGGL((ftk::grad_accumulate_finish_kernel<AT, GT, ZERO, STATS>), dim3(1), dim3(256), 0, stream, acc, g,
                            static_cast<uint64_t>(head), static_cast<uint64_t>(tail_begin), static_cast<uint64_t>(n),
                            scale, pre_mult, static_cast<const ftk::StatsPartial*>(parts), reduce_blocks, stats_out,
-                           stats_accumulate);
+                           stats_accumulate, dec.inv_scale, dec.max_norm, dec.ctl);
         FT_HIP(hipGetLastError());
     }
     return FT_OK;
@@ -443,22 +450,22 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
 
 template <int AT, int GT>
 int launch_accumulate_flags(bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec, float scale,
-                            float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, hipStream_t stream)
+                            float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, const Decide& dec, hipStream_t stream)
 {
-    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
-    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
-    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
-    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
+    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
 }
 
 template <int AT>
 int launch_accumulate_g(int g_dtype, bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec,
-                        float scale, float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, hipStream_t stream)
+                        float scale, float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, const Decide& dec, hipStream_t stream)
 {
     switch (g_dtype) {
-        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
-        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
-        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, stream);
+        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
     }
 }
 
@@ -610,8 +617,12 @@ size_t ft_grad_stats_workspace_bytes(void) { return sizeof(ftk::StatsPartial) * 
 
 size_t ft_grad_accumulate_workspace_bytes(size_t n) { return accumulate_workspace_bytes(n); }
 
-int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate, void* workspace,
-                  size_t workspace_bytes, void* stream_)
+}  // extern "C"
+
+namespace {
+
+int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate, void* workspace,
+                    size_t workspace_bytes, const Decide& dec, void* stream_)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (!out) return fth::fail(FT_EINVAL, "out must not be NULL");
@@ -662,19 +673,41 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
     switch (g_dtype) {
         case FT_F32:
             hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate);
+                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl);
             break;
         case FT_F16:
             hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate);
+                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl);
             break;
         default:
             hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_BF16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate);
+                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl);
             break;
     }
     FT_HIP(hipGetLastError());
     return FT_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate, void* workspace,
+                  size_t workspace_bytes, void* stream)
+{
+    return grad_stats_impl(g, g_dtype, n, pre_mult, out, accumulate, workspace, workspace_bytes, Decide{}, stream);
+}
+
+int ft_grad_decide(const void* g, int g_dtype, size_t n, float pre_mult, void* stats, int accumulate, float inv_scale,
+                   float max_norm, void* ctl_out, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!ctl_out) return fth::fail(FT_EINVAL, "ctl_out must not be NULL");
+    if (!aligned(ctl_out, 16)) return fth::fail(FT_EALIGN, "ft_step_control_t must be 16-byte aligned");
+    Decide dec;
+    dec.inv_scale = inv_scale;
+    dec.max_norm = max_norm;
+    dec.ctl = static_cast<ft_step_control_t*>(ctl_out);
+    return grad_stats_impl(g, g_dtype, n, pre_mult, stats, accumulate, workspace, workspace_bytes, dec, stream);
 }
 
 }  // extern "C"
@@ -685,7 +718,7 @@ namespace {
 // allocated); otherwise the caller's workspace, or the library-owned buffer when that is NULL.
 int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
                          float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
-                         size_t workspace_bytes, bool static_scratch_only, void* stream_)
+                         size_t workspace_bytes, bool static_scratch_only, const Decide& dec, void* stream_)
 {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (!valid_dtype(acc_dtype) || !valid_dtype(g_dtype))
@@ -715,9 +748,9 @@ int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t 
     }
     ft_grad_stats_t* out = static_cast<ft_grad_stats_t*>(stats_out);
     switch (acc_dtype) {
-        case FT_F32: return launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
-        case FT_F16: return launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
-        default: return launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, stream);
+        case FT_F32: return launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
+        case FT_F16: return launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
+        default: return launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
     }
 }
 
@@ -730,7 +763,21 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
                        size_t workspace_bytes, void* stream)
 {
     return grad_accumulate_impl(acc, acc_dtype, g, g_dtype, n, scale, zero_g, stats_pre_mult, stats_out, stats_accumulate,
-                                workspace, workspace_bytes, false, stream);
+                                workspace, workspace_bytes, false, Decide{}, stream);
+}
+
+int ft_grad_accumulate_decide(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                              float stats_pre_mult, void* stats, int stats_accumulate, float inv_scale, float max_norm,
+                              void* ctl_out, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!stats || !ctl_out) return fth::fail(FT_EINVAL, "stats and ctl_out must not be NULL");
+    if (!aligned(ctl_out, 16)) return fth::fail(FT_EALIGN, "ft_step_control_t must be 16-byte aligned");
+    Decide dec;
+    dec.inv_scale = inv_scale;
+    dec.max_norm = max_norm;
+    dec.ctl = static_cast<ft_step_control_t*>(ctl_out);
+    return grad_accumulate_impl(acc, acc_dtype, g, g_dtype, n, scale, zero_g, stats_pre_mult, stats, stats_accumulate,
+                                workspace, workspace_bytes, false, dec, stream);
 }
 
 int ft_grad_accumulate_static(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
@@ -741,7 +788,7 @@ int ft_grad_accumulate_static(void* acc, int acc_dtype, void* g, int g_dtype, si
                          "(use ft_grad_accumulate with a workspace for longer buffers)",
                          static_cast<unsigned long long>(FT_STATIC_MAX_ELEMS), n);
     return grad_accumulate_impl(acc, acc_dtype, g, g_dtype, n, scale, zero_g, stats_pre_mult, stats_out, stats_accumulate,
-                                nullptr, 0, true, stream);
+                                nullptr, 0, true, Decide{}, stream);
 }
 
 int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ctl_out, void* stream)

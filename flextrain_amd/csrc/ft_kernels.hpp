@@ -473,13 +473,47 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
     block_stats_epilogue<BLOCK>(lane_sum, bad, partials);
 }
 
+// The per-step decision from a statistics record (one thread):
+//   skip = nonfinite != 0 . norm = sqrt(sumsq) (double) . clip = min(1, max_norm / (norm + 1e-6))
+//   (double, then fp32; 1 when max_norm <= 0) . grad_mult = clip * inv_scale (one fp32 multiply)
+__device__ __forceinline__ void write_decision(uint64_t nonfinite, double sumsq, float inv_scale, float max_norm,
+                                               ft_step_control_t* ctl)
+{
+    const double norm = __builtin_sqrt(sumsq);
+    double coef = 1.0;
+    if (max_norm > 0.0f) {
+        coef = (double)max_norm / (norm + 1e-6);
+        if (!(coef < 1.0)) coef = 1.0;
+    }
+    const float clip = (float)coef;
+    ctl->skip = nonfinite != 0 ? 1u : 0u;
+    ctl->grad_mult = clip * inv_scale;
+    ctl->grad_norm = (float)norm;
+    ctl->clip_coef = clip;
+}
+
+// Stores (or adds to) the statistics record and, when a control record is asked for, decides from
+// the record as it now stands: the last launch of a statistics pass then is the decision as well.
+__device__ __forceinline__ void publish_stats(double s, uint64_t b, ft_grad_stats_t* out, int accumulate, float inv_scale,
+                                              float max_norm, ft_step_control_t* ctl)
+{
+    if (accumulate) {
+        s += out->sumsq;
+        b += out->nonfinite;
+    }
+    out->sumsq = s;
+    out->nonfinite = b;
+    if (ctl) write_decision(b, s, inv_scale, max_norm, ctl);
+}
+
 // Stage 2 (one block of 256): adds the block partials in a fixed tree order, then the up to
 // `edge` elements before/after the vector body one by one, and writes or accumulates the result.
 template <int GT>
 __global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartial* __restrict__ partials,
                                                                int nparts, const void* g, uint64_t head,
                                                                uint64_t tail_begin, uint64_t n, float pre_mult,
-                                                               ft_grad_stats_t* out, int accumulate)
+                                                               ft_grad_stats_t* out, int accumulate, float inv_scale,
+                                                               float max_norm, ft_step_control_t* ctl)
 {
     __shared__ double s_sum[256];
     __shared__ uint64_t s_bad[256];
@@ -524,13 +558,7 @@ __global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartia
                 s += (double)u * (double)u;
             }
         }
-        if (accumulate) {
-            out->sumsq += s;
-            out->nonfinite += b;
-        } else {
-            out->sumsq = s;
-            out->nonfinite = b;
-        }
+        publish_stats(s, b, out, accumulate, inv_scale, max_norm, ctl);
     }
 }
 
@@ -685,7 +713,8 @@ __global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, 
                                                                      uint64_t tail_begin, uint64_t n, float scale,
                                                                      float pre_mult,
                                                                      const StatsPartial* __restrict__ partials,
-                                                                     int nparts, ft_grad_stats_t* out, int accumulate)
+                                                                     int nparts, ft_grad_stats_t* out, int accumulate,
+                                                                     float inv_scale, float max_norm, ft_step_control_t* ctl)
 {
     double s = 0.0;
     uint64_t b = 0;
@@ -751,13 +780,7 @@ __global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, 
         if (threadIdx.x == 0) {
             s += s_sum[0];
             b += s_bad[0];
-            if (accumulate) {
-                out->sumsq += s;
-                out->nonfinite += b;
-            } else {
-                out->sumsq = s;
-                out->nonfinite = b;
-            }
+            publish_stats(s, b, out, accumulate, inv_scale, max_norm, ctl);
         }
     }
 }
@@ -766,17 +789,7 @@ __global__ void grad_control_kernel(const ft_grad_stats_t* stats, float inv_scal
                                     ft_step_control_t* ctl)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    const double norm = __builtin_sqrt(stats->sumsq);
-    double coef = 1.0;
-    if (max_norm > 0.0f) {
-        coef = (double)max_norm / (norm + 1e-6);
-        if (!(coef < 1.0)) coef = 1.0;
-    }
-    const float clip = (float)coef;
-    ctl->skip = stats->nonfinite != 0 ? 1u : 0u;
-    ctl->grad_mult = clip * inv_scale;
-    ctl->grad_norm = (float)norm;
-    ctl->clip_coef = clip;
+    write_decision(stats->nonfinite, stats->sumsq, inv_scale, max_norm, ctl);
 }
 
 }  // namespace ftk

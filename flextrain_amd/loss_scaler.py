@@ -196,6 +196,25 @@ class GradientGuard:
                 0 if self._fresh else 1, self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(grads.device)))
         self._fresh = False
 
+    def add_and_decide(self, grads: torch.Tensor, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``add(grads)`` followed by ``decide_async(...)`` with one launch fewer: the kernel that
+        finishes the statistics writes the decision as well. For the last (or only) gradient buffer
+        of a step. Returns the control record like ``decide_async``."""
+        if not grads.is_cuda or not grads.is_contiguous():
+            raise ValueError("gradients must be a contiguous GPU tensor")
+        target = self.control if out is None else out
+        if out is not None and (not out.is_cuda or out.numel() * out.element_size() < 16 or out.data_ptr() % 16):
+            raise ValueError("out must be 16 bytes of 16-byte aligned device memory")
+        inv_scale = float(1.0 / float(loss_scale))
+        with torch.cuda.device(grads.device):
+            _C.check("ft_grad_decide", self._lib.ft_grad_decide(
+                grads.data_ptr(), _C.dtype_code(grads.dtype), grads.numel(), inv_scale, self.stats_ptr,
+                0 if self._fresh else 1, inv_scale, float(max_grad_norm) if max_grad_norm else 0.0, target.data_ptr(),
+                self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(grads.device)))
+        self._fresh = False
+        return target
+
     def accumulate(self, acc: torch.Tensor, grads: torch.Tensor, scale: float = 1.0, zero_grads: bool = False,
                    with_stats: bool = False, loss_scale: float = 1.0) -> None:
         """``acc += scale * grads`` in one pass (one fused multiply-add per element, rounded to

@@ -88,9 +88,9 @@ class FlexTrainCPUOptimizer(ABC):
                 if guard is None or guard.device != live[0].device:
                     guard = self._step_guard = GradientGuard(live[0].device)
                 guard.begin()
-                for g in live:
+                for g in live[:-1]:
                     guard.add(g, loss_scale=loss_scale)
-                extensions["control"] = guard.decide_async(loss_scale=loss_scale, max_grad_norm=max_grad_norm)
+                extensions["control"] = guard.add_and_decide(live[-1], loss_scale=loss_scale, max_grad_norm=max_grad_norm)
         elif loss_scale != 1.0:
             if "control" in extensions:
                 raise ValueError("loss_scale is already part of the control record passed in")
@@ -345,8 +345,7 @@ class FlexTrainOptimizer:
                 self._guard = GradientGuard(device=grads.device)
             scale = float(self.loss_scaler.loss_scale) if self.loss_scaler is not None else 1.0
             self._guard.begin()
-            self._guard.add(grads, loss_scale=scale)
-            extensions["control"] = self._guard.decide_async(loss_scale=scale, max_grad_norm=self.max_grad_norm)
+            extensions["control"] = self._guard.add_and_decide(grads, loss_scale=scale, max_grad_norm=self.max_grad_norm)
         self.cpu_optimizer.step(self.non_layerwise_step_contexts, **extensions)
         self._zero_grads()
         if self._offload and self._device_dtype == self._master_dtype:

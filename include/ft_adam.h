@@ -146,6 +146,16 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
                        float stats_pre_mult, void* stats_out, int stats_accumulate, void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/* ft_grad_decide / ft_grad_accumulate_decide: ft_grad_stats / ft_grad_accumulate (with statistics)
+ * followed by ft_grad_control on the record as it then stands, without the extra launch: the last
+ * kernel of the statistics pass writes the decision too. For the pass that completes a step's
+ * statistics (the last gradient buffer, the last micro-batch). Same results as the two calls. */
+int ft_grad_decide(const void* g, int g_dtype, size_t n, float pre_mult, void* stats, int accumulate, float inv_scale,
+                   float max_norm, void* ctl_out, void* workspace, size_t workspace_bytes, void* stream);
+int ft_grad_accumulate_decide(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
+                              float stats_pre_mult, void* stats, int stats_accumulate, float inv_scale, float max_norm,
+                              void* ctl_out, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ft_grad_accumulate_static: ft_grad_accumulate for callers that cannot allocate (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc). No counterpart in the
  * reference. Same arguments, results and kernels as ft_grad_accumulate, without the workspace: the

@@ -288,3 +288,41 @@ def test_library_owned_scratch_is_per_stream(cuda, oracle):
         bad, sumsq = oracle.grad_stats(_bits(grads[k][0]), CODE[torch.bfloat16], pre_mult=0.5)
         got = records[k][2].cpu()  # acc was zero: the accumulated values are the gradients, widened
         assert int(got[0:1].view(torch.int64).item()) == bad and abs(float(got[1]) - sumsq) <= 2 * NORM_RTOL * sumsq
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_fused_decision_equals_statistics_then_control(cuda, dtype):
+    """ft_grad_decide / ft_grad_accumulate_decide against ft_grad_stats / ft_grad_accumulate followed
+    by ft_grad_control: the same record and the same decision, bit for bit, also when the pass adds
+    to an existing record and when an inf is present."""
+    from flextrain_amd import _C
+    from flextrain_amd.loss_scaler import GradientGuard
+    lib = _C.lib()
+    n = 1_234_567
+    gen = torch.Generator(device=cuda).manual_seed(31)
+    grads = [(torch.randn(n, device=cuda, generator=gen) * 37.0).to(dtype) for _ in range(3)]
+    grads[2][n // 3] = float("inf")
+    a, b = GradientGuard(cuda), GradientGuard(cuda)
+    for g in grads:  # the record grows over the three buffers; decide after each
+        a.add(g, loss_scale=64.0)
+        a.decide_async(loss_scale=64.0, max_grad_norm=2.0)
+        b.add_and_decide(g, loss_scale=64.0, max_grad_norm=2.0)
+        torch.cuda.synchronize()
+        assert a._buf.cpu().view(torch.int64).tolist() == b._buf.cpu().view(torch.int64).tolist()
+    assert b.read().overflow and b.read().nonfinite == 1
+    # the accumulation pass
+    acc_a, acc_b = torch.zeros(n, device=cuda), torch.zeros(n, device=cuda)
+    ws = torch.empty(int(lib.ft_grad_accumulate_workspace_bytes(n)), dtype=torch.uint8, device=cuda)
+    rec_a, rec_b = torch.zeros(4, dtype=torch.float64, device=cuda), torch.zeros(4, dtype=torch.float64, device=cuda)
+    stream = _C.current_stream_ptr(cuda)
+    g = grads[0]
+    code = _C.dtype_code(dtype)
+    _C.check("ft_grad_accumulate", lib.ft_grad_accumulate(acc_a.data_ptr(), _C.F32, g.data_ptr(), code, n, 0.5, 0, 1 / 64.0,
+                                                          rec_a.data_ptr(), 0, ws.data_ptr(), ws.numel(), stream))
+    _C.check("ft_grad_control", lib.ft_grad_control(rec_a.data_ptr(), 1 / 64.0, 2.0, rec_a[2:].data_ptr(), stream))
+    _C.check("ft_grad_accumulate_decide", lib.ft_grad_accumulate_decide(
+        acc_b.data_ptr(), _C.F32, g.data_ptr(), code, n, 0.5, 0, 1 / 64.0, rec_b.data_ptr(), 0, 1 / 64.0, 2.0, rec_b[2:].data_ptr(),
+        ws.data_ptr(), ws.numel(), stream))
+    torch.cuda.synchronize()
+    assert torch.equal(acc_a, acc_b) and rec_a.cpu().view(torch.int64).tolist() == rec_b.cpu().view(torch.int64).tolist()
+    assert float(rec_b.cpu()[2:].view(torch.float32)[3]) < 1.0  # clipped: the decision really was taken
