@@ -28,7 +28,8 @@ N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 8
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
 # profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_657_000, "cfg3": 5_666_664_000, "cfg4": 23_958_221_000, "accumulate": 2_453_887_000}
+MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_664_000, "cfg3": 5_666_664_000, "cfg4": 23_958_221_000, "accumulate": 2_453_887_000,
+                          "multi": 5_666_716_000}
 # The summary each literal is copied from; it carries the line "roofline.traffic = <bytes> B"
 # (tests/test_bench_contract.py checks that the two agree).
 TRAFFIC_SOURCE = {
@@ -36,6 +37,7 @@ TRAFFIC_SOURCE = {
     "cfg3": "profiles/grad_stats_and_adam_cfg3_overflow_path.md",
     "cfg4": "profiles/adam_tile_kernel_cfg4_llama70b_layer.md",
     "accumulate": "profiles/grad_accumulate_kernel_llama7b_layer.md",
+    "multi": "profiles/adam_multi_kernel_cfg2_partition_16_ragged_contexts.md",
 }
 
 HP = dict(lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, bias_correction=True)
@@ -504,6 +506,12 @@ def bench_multi(args, torch, dev) -> int:
     n, k = N_7B_LAYER, max(1, args.segments)
     eng = FlexTrainCPUAdam(**HP)
     p, g, m, v, h = make_inputs(torch, n, torch.bfloat16, 1e-3, dev)
+    if args.calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
+        scratch = torch.empty_like(p)
+        for _ in range(3):
+            scratch.copy_(p)
+        torch.cuda.synchronize()
+        del scratch
     rng = random.Random(0)
     cuts = sorted({0, n} | {rng.randrange(1, n) for _ in range(k - 1)})
     groups = [dict(HP, step=100), dict(HP, step=37, weight_decay=0.0)]
@@ -546,7 +554,10 @@ def bench_multi(args, torch, dev) -> int:
                                "stepped by one launch (against one call per context)", "elements": n, "segments": len(ctxs),
                    "shortest": min(c.full_parameter.numel() for c in ctxs), "longest": max(c.full_parameter.numel() for c in ctxs)},
         "roofline": {"bound": "hbm", "kernel": "adam_multi_kernel", "achieved": main["achieved_gbps"], "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": main["frac"], "traffic": None, "algorithmic_bytes_per_launch": n * 28,
+                     "unit": "GB/s", "frac": main["frac"],
+                     "traffic": MEASURED_TRAFFIC_BYTES["multi"] if len(ctxs) == 16 else None,
+                     "traffic_source": TRAFFIC_SOURCE["multi"] if len(ctxs) == 16 else None,
+                     "algorithmic_bytes_per_launch": n * 28,
                      "kernel_ms_avg": main["ms_avg"]},
         "variants": results,
     }), flush=True)
