@@ -20,7 +20,9 @@
  * Pinned by (see tests/): bit-exact agreement with the compiled reference (oracle/_ref) on
  * committed golden vectors and on fresh random inputs, closed forms at t=1 with m=v=0,
  * invariants (g=m=v=0), torch.optim.AdamW to ~1e-6, and for the conversions brute force against
- * numpy / torch casts.
+ * numpy / torch casts. ft_oracle_adam_trace: every intermediate against exact rational arithmetic
+ * rounded once per operation, for the three weight-decay modes, and its p', m', v' against
+ * ft_oracle_adam_step. No function of the checker is without such a check.
  *
  * Extensions with NO counterpart in the reference (the reference never unscales, checks or
  * clips gradients -- flextrain/engine.py:249 multiplies the loss and nothing divides the
