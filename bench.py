@@ -429,6 +429,7 @@ def bench_pipeline(args, torch, dev) -> int:
                                "fp32 state in pinned host DRAM, bf16 grads and parameters on GPU",
                    "elements": total, "units": units, "micro_batches": mb, "chunk_elems": args.chunk_elems,
                    "slots": args.slots, "unit_windows": args.windows},
+        "iteration_ms": [w * 1e3 for w in walls],
         "link": dict(link, achieved_each_way_gbps=one_way, achieved_total_gbps=2 * one_way,
                      frac_of_unidirectional=one_way / link["unidirectional_ceiling_gbps"],
                      frac_of_bidirectional_measured=2 * one_way / link["bidirectional_sum_measured_gbps"]),
