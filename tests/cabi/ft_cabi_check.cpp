@@ -185,6 +185,118 @@ void accumulate_pass(hipStream_t stream)
     HIP_OK(hipFree(dacc)); HIP_OK(hipFree(dg)); HIP_OK(hipFree(ws)); HIP_OK(hipFree(rec));
 }
 
+// Many step contexts in one call: three ragged segments of two "parameter groups" (different
+// learning rate, decay and step) cut out of flat buffers at odd element offsets, statistics and
+// decision in one fused call (ft_grad_decide) over the whole gradient buffer.
+void many_segments_one_launch(hipStream_t stream)
+{
+    const size_t total = 700011;
+    const size_t lo[3] = {1, 200002, 200007}, len[3] = {200000, 5, 500001};
+    const float lr[3] = {LR, 3e-4f, LR}, wd[3] = {WD, 0.f, WD};
+    const uint64_t step[3] = {10, 4, 10};
+    Rng rng{5};
+    std::vector<float> p(total), m(total), v(total);
+    std::vector<uint16_t> g(total), h(total, 0x4111);
+    for (size_t i = 0; i < total; ++i) {
+        p[i] = rng.normal(0.02f);
+        m[i] = rng.normal(1e-4f);
+        v[i] = (float)(rng.uniform() * 1e-6);
+        g[i] = ft_oracle_f32_to_bf16(rng.normal(1e-3f) * 8.f);
+    }
+    float *dp = dev_copy(p), *dm = dev_copy(m), *dv = dev_copy(v);
+    uint16_t *dg = dev_copy(g), *dh = dev_copy(h);
+    void* ws = nullptr;
+    char* rec = nullptr;
+    HIP_OK(hipMalloc(&ws, ft_grad_stats_workspace_bytes()));
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&rec), 32));
+    FT_OK_OR_DIE(ft_adam_create(9, LR, B1, B2, EPS, WD, 1, 0));
+    FT_OK_OR_DIE(ft_grad_decide(dg, FT_BF16, total, 1.f / 8.f, rec, 0, 1.f / 8.f, 0.f, rec + 16, ws, ft_grad_stats_workspace_bytes(), stream));
+    ft_adam_segment_t segs[3];
+    std::memset(segs, 0, sizeof segs);
+    for (int k = 0; k < 3; ++k) {
+        segs[k].p = dp + lo[k];
+        segs[k].g = dg + lo[k];
+        segs[k].m = dm + lo[k];
+        segs[k].v = dv + lo[k];
+        segs[k].half_out = dh + lo[k];
+        segs[k].n = len[k];
+        segs[k].step = step[k];
+        segs[k].lr = lr[k];
+        segs[k].beta1 = B1;
+        segs[k].beta2 = B2;
+        segs[k].eps = EPS;
+        segs[k].weight_decay = wd[k];
+        segs[k].bias_correction = 1;
+        segs[k].grad_mult = 123.f;  // overridden by the control record
+    }
+    FT_OK_OR_DIE(ft_adam_step_multi(9, segs, 3, FT_BF16, FT_BF16, rec + 16, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    ft_step_control_t ctl;
+    HIP_OK(hipMemcpy(&ctl, rec + 16, 16, hipMemcpyDeviceToHost));
+    check(ctl.skip == 0 && ctl.grad_mult == 1.f / 8.f && ctl.clip_coef == 1.f, "fused statistics + decision: unscale only");
+    for (int k = 0; k < 3; ++k) {
+        ft_oracle_scalars s;
+        ft_oracle_scalars_compute(step[k], lr[k], B1, B2, EPS, wd[k], 1, 1, 0, &s);
+        ft_oracle_adam_step(&s, ctl.grad_mult, p.data() + lo[k], g.data() + lo[k], FT_ORACLE_BF16, m.data() + lo[k], v.data() + lo[k],
+                            h.data() + lo[k], FT_ORACLE_BF16, len[k], -1, 0);
+    }
+    check(same_bits(dp, p) && same_bits(dm, m) && same_bits(dv, v) && same_bits(dh, h),
+          "many segments: every segment bit-identical to the CPU checker, nothing outside them touched");
+    segs[1].m = nullptr;
+    check(ft_adam_step_multi(9, segs, 3, FT_BF16, FT_BF16, nullptr, stream) == FT_EINVAL, "many segments: a NULL array is refused");
+    HIP_OK(hipStreamSynchronize(stream));
+    check(same_bits(dp, p), "many segments: a refused call launched nothing");
+    FT_OK_OR_DIE(ft_adam_destroy(9));
+    HIP_OK(hipFree(dp)); HIP_OK(hipFree(dm)); HIP_OK(hipFree(dv)); HIP_OK(hipFree(dg)); HIP_OK(hipFree(dh)); HIP_OK(hipFree(ws)); HIP_OK(hipFree(rec));
+}
+
+// The accumulation pass without any workspace: the library's static scratch.
+void accumulate_without_allocating(hipStream_t stream)
+{
+    const size_t n = 400003;
+    Rng rng{11};
+    std::vector<float> acc(n);
+    std::vector<uint16_t> g(n);
+    for (size_t i = 0; i < n; ++i) {
+        acc[i] = rng.normal(1.f);
+        g[i] = ft_oracle_f32_to_f16(rng.normal(0.1f));
+    }
+    float* dacc = dev_copy(acc);
+    uint16_t* dg = dev_copy(g);
+    char* rec = nullptr;
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&rec), 16));
+    size_t free_before = 0, free_after = 0, total = 0;
+    FT_OK_OR_DIE(ft_grad_accumulate_static(dacc, FT_F32, dg, FT_F16, 16, 1.0f, 0, 1.0f, rec, 0, stream));  // first use on this device
+    HIP_OK(hipStreamSynchronize(stream));
+    ft_oracle_grad_accumulate(acc.data(), FT_ORACLE_F32, g.data(), FT_ORACLE_F16, 16, 1.0f, 0);
+    HIP_OK(hipMemGetInfo(&free_before, &total));
+    FT_OK_OR_DIE(ft_grad_accumulate_static(dacc, FT_F32, dg, FT_F16, n, 0.5f, 0, 1.0f, rec, 0, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemGetInfo(&free_after, &total));
+    ft_oracle_grad_accumulate(acc.data(), FT_ORACLE_F32, g.data(), FT_ORACLE_F16, n, 0.5f, 0);
+    check(same_bits(dacc, acc), "static scratch: acc bit-identical to the CPU checker");
+    ft_grad_stats_t stats;
+    HIP_OK(hipMemcpy(&stats, rec, 16, hipMemcpyDeviceToHost));
+    uint64_t bad = 0;
+    double sumsq = 0;
+    ft_oracle_grad_stats(acc.data(), FT_ORACLE_F32, n, 1.0f, &bad, &sumsq, 0);
+    check(stats.nonfinite == 0 && std::fabs(stats.sumsq - sumsq) <= 2e-6 * sumsq, "static scratch: fused statistics match");
+    check(free_before == free_after, "static scratch: the call changed nothing about device memory");
+    check(ft_grad_accumulate_static(dacc, FT_F32, dg, FT_F16, (size_t)FT_STATIC_MAX_ELEMS + 1, 1.f, 0, 1.f, rec, 0, stream) == FT_EINVAL,
+          "static scratch: more than the maximum is refused");
+    HIP_OK(hipFree(dacc)); HIP_OK(hipFree(dg)); HIP_OK(hipFree(rec));
+}
+
+void link_probe()
+{
+    ft_link_probe_t r;
+    FT_OK_OR_DIE(ft_link_probe(64u << 20, 2, &r));
+    std::printf("link: copies %.1f / %.1f / %.1f GB/s, copy kernel %.1f / %.1f / %.1f GB/s (H2D / D2H / both)\n", r.h2d_copy, r.d2h_copy,
+                r.both_copy, r.h2d_kernel, r.d2h_kernel, r.both_kernel);
+    check(r.h2d_copy > 1 && r.d2h_copy > 1 && r.both_copy > 1 && r.h2d_kernel > 1 && r.d2h_kernel > 1 && r.both_kernel > 1,
+          "link probe: six figures, all positive");
+}
+
 void offloaded_step(hipStream_t stream)
 {
     const size_t n = 3 * (1u << 18) + 1001;  // four chunks, the last one partial
@@ -268,7 +380,10 @@ int main()
     HIP_OK(hipStreamCreate(&stream));
     resident_mixed_precision_step(stream);
     accumulate_pass(stream);
+    many_segments_one_launch(stream);
+    accumulate_without_allocating(stream);
     offloaded_step(stream);
+    link_probe();
     synthetic_inputs(stream);
     HIP_OK(hipStreamDestroy(stream));
     std::printf("%s (%d failed)\n", g_failures ? "FAILED" : "ALL PASSED", g_failures);
