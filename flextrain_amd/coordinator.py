@@ -182,6 +182,7 @@ class FlexTrainOptsCoordinator:
         self._iteration_open = False  # statistics of the running iteration have been started
         self._pending_steps = False   # deferred schedule: a decision has been taken and not yet applied
         self._deferred_skip = False
+        self._deferred_grad_mult = 1.0
         self.last_decision = None
         self.last_skipped_units: List[int] = []
         if self._guarded:
@@ -306,7 +307,8 @@ class FlexTrainOptsCoordinator:
         if self._guarded:  # skip and the gradient multiplier come from the unit's device-side record
             extensions["control"] = self._unit_controls[self._num_units if self._defer else unit_index]
         elif self._loss_scaler is not None:
-            extensions["grad_mult"] = float(1.0 / self.loss_scale)
+            # deferred: the scale the gradients were produced under, not what the scaler holds by now
+            extensions["grad_mult"] = self._deferred_grad_mult if self._defer else float(1.0 / self.loss_scale)
         if self._offload:
             self._optimizer.cpu_optimizer.step(contexts, blocking=False, guard_stream=False, **extensions)
             if micro_batch_index == self._micro_batch_per_rank - 1 and unit_index in self._open_windows:
@@ -411,6 +413,7 @@ class FlexTrainOptsCoordinator:
             if self._guarded:
                 self._iter_guard.decide_async(loss_scale=self.loss_scale, max_grad_norm=self._max_grad_norm,
                                               out=self._unit_controls[self._num_units])
+            self._deferred_grad_mult = float(1.0 / self.loss_scale)
             decision = self._finish_iteration_statistics()
             self._pending_steps = True
             self._deferred_skip = bool(decision.overflow) if decision is not None else False
@@ -481,6 +484,8 @@ class FlexTrainOptsCoordinator:
         share, so there is no ``.0`` file, as for any empty share in the reference). Waits for the
         steps in flight first. Returns the paths."""
         from .state_files import BACKWARD_SHARE, write_unit_opts
+        if self._defer and self._pending_steps:
+            raise RuntimeError("a decided iteration has not been applied yet; save after the forward-side hooks have run")
         if self._open_windows:
             raise RuntimeError("units %s are being stepped on the GPU; save after clear_backward_pipeline()" % sorted(self._open_windows))
         self.synchronize()
