@@ -375,7 +375,7 @@ def bench_pipeline(args, torch, dev) -> int:
     n, mb = N_7B_LAYER, args.micro_batches
     if args.resident:
         return bench_pipeline_resident(args, torch, dev, Unit)
-    units = min(args.layers, 24)  # 24 layers = 58 GB of pinned state, inside what the box pins
+    units = min(args.layers, 24 + args.resident_units)  # 24 streamed layers = 58 GB of pinned state, inside what the box pins
     coord = None
     while coord is None:
         flat = [(torch.randn(n, device=dev) * 0.02).to(torch.bfloat16) for _ in range(units)]
@@ -388,7 +388,8 @@ def bench_pipeline(args, torch, dev) -> int:
             coord = FlexTrainOptsCoordinator()
             coord.initialize(opt, flat, mb, offload=True,
                              unit_windows={"auto": None, "off": False}.get(args.windows, True),
-                             window_write_through=args.windows == "write_through")
+                             window_write_through=args.windows == "write_through",
+                             resident_units=args.resident_units)
         except _C.FtError:
             coord = None
             del opt, flat, params
@@ -421,7 +422,8 @@ def bench_pipeline(args, torch, dev) -> int:
         walls.append(time.perf_counter() - t0)
     sec = sum(walls) / len(walls)
     total = units * n
-    one_way = total * 12 / sec / 1e9
+    streamed = (units - min(args.resident_units, units)) * n
+    one_way = streamed * 12 / sec / 1e9
     print(json.dumps({
         "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
         "value": total / sec, "unit": "elements/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -430,7 +432,8 @@ def bench_pipeline(args, torch, dev) -> int:
         "config": {"workload": f"pipeline: coordinator schedule over {units} Llama-7B layers, {mb} shares per unit, "
                                "fp32 state in pinned host DRAM, bf16 grads and parameters on GPU",
                    "elements": total, "units": units, "micro_batches": mb, "chunk_elems": args.chunk_elems,
-                   "slots": args.slots, "unit_windows": args.windows},
+                   "slots": args.slots, "unit_windows": args.windows, "resident_units": min(args.resident_units, units),
+                   "streamed_elements": streamed},
         "iteration_ms": [w * 1e3 for w in walls],
         "link": dict(link, achieved_each_way_gbps=one_way, achieved_total_gbps=2 * one_way,
                      frac_of_unidirectional=one_way / link["unidirectional_ceiling_gbps"],
@@ -637,6 +640,8 @@ def main() -> int:
     ap.add_argument("--chunk-elems", type=int, default=64 * 1024 * 1024, help="cfg5: elements per streamed chunk")
     ap.add_argument("--slots", type=int, default=3, help="cfg5: device buffer sets of the pipeline")
     ap.add_argument("--layers", type=int, default=32, help="cfg5: decoder layers (32 = the full 7B optimizer)")
+    ap.add_argument("--resident-units", type=int, default=0,
+                    help="pipeline: units whose fp32 state stays in HBM although the others are streamed from host memory")
     ap.add_argument("--resident", action="store_true",
                     help="pipeline: keep the fp32 state of every unit in HBM instead of pinned host memory")
     ap.add_argument("--no-cpu-baseline", action="store_true")

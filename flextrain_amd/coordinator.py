@@ -92,6 +92,7 @@ class FlexTrainOptsCoordinator:
         offload: bool = True,
         unit_windows: Optional[bool] = None,
         window_write_through: bool = False,
+        resident_units: int = 0,
         loss_scaler=None,
         check_overflow: Optional[bool] = None,
         max_grad_norm: Optional[float] = None,
@@ -124,6 +125,13 @@ class FlexTrainOptsCoordinator:
             window_write_through: a window's results are written to the host by the step kernels
                 themselves instead of being copied back in one piece after the unit's last share
                 (slower: 43.7 GB/s on the same schedule).
+            resident_units: with ``offload``, keep the master state of units ``0 .. resident_units-1``
+                in HBM all the same and stream only the others. Those are the units stepped last in
+                an iteration (and needed first by the next forward pass), where no backward work is
+                left to hide their transfers behind; every resident unit takes 12 bytes per
+                element each way off the host link. The reference keeps all optimizer state on
+                the host (``:133-136`` refuses a GPU optimizer); with 288 GB of HBM how much to
+                offload is a dial, not a yes or no.
             loss_scaler: object with ``loss_scale`` and ``update_scale(overflow)``
                 (``flextrain_amd.loss_scaler``): the gradients were produced from
                 ``loss * loss_scale`` and are divided by it inside the update.
@@ -150,9 +158,12 @@ class FlexTrainOptsCoordinator:
         self._micro_batch_per_rank = micro_batch_per_rank
         self._unit_half_parameters = units
         self._offload = bool(offload)
+        resident_units = max(0, min(int(resident_units), self._num_units)) if self._offload else self._num_units
+        self._unit_resident = [u < resident_units for u in range(self._num_units)]
         if unit_windows is None:
             share_numel = self._unit_numel // micro_batch_per_rank
-            unit_windows = not (share_numel >= 32 * 1024 * 1024 and self._num_units * micro_batch_per_rank <= 96)
+            streamed_units = self._num_units - sum(self._unit_resident)
+            unit_windows = not (share_numel >= 32 * 1024 * 1024 and streamed_units * micro_batch_per_rank <= 96)
         self._unit_windows = bool(unit_windows) and self._offload
         self._open_windows = {}  # unit index -> window token
         self._window_write_through = bool(window_write_through)
@@ -212,9 +223,10 @@ class FlexTrainOptsCoordinator:
 
         # [master | exp_avg | exp_avg_sq] per unit.
         per_element = 1 + optimizer.optimizer_state_per_element
-        state_device = torch.device("cpu") if self._offload else device
-        self._unit_opts = allocate_memory_chunks(
-            self._unit_numel, (self._num_units, per_element), master_dtype, state_device)
+        self._unit_opts = [
+            list(allocate_memory_chunks(self._unit_numel, per_element, master_dtype,
+                                        device if self._unit_resident[u] else torch.device("cpu")))
+            for u in range(self._num_units)]
 
         # Seed the master copy from the low-precision parameters (exact: widening conversion).
         for u in range(self._num_units):
@@ -292,7 +304,8 @@ class FlexTrainOptsCoordinator:
         copies run while the previous unit is still being stepped."""
         if self._defer and self._deferred_skip:
             return
-        if self._unit_windows and not self._is_invalid_unit(unit_index) and unit_index not in self._open_windows:
+        if self._unit_windows and not self._is_invalid_unit(unit_index) and not self._unit_resident[unit_index] \
+                and unit_index not in self._open_windows:
             self._open_windows[unit_index] = self._optimizer.cpu_optimizer.open_window(*self._unit_opts[unit_index], write_through=self._window_write_through)
 
     def _execute_optimizer_step(self, unit_index: int, micro_batch_index: int) -> None:
@@ -309,12 +322,12 @@ class FlexTrainOptsCoordinator:
         elif self._loss_scaler is not None:
             # deferred: the scale the gradients were produced under, not what the scaler holds by now
             extensions["grad_mult"] = self._deferred_grad_mult if self._defer else float(1.0 / self.loss_scale)
-        if self._offload:
+        if self._unit_resident[unit_index]:
+            self._optimizer.cpu_optimizer.step(contexts, **extensions)
+        else:
             self._optimizer.cpu_optimizer.step(contexts, blocking=False, guard_stream=False, **extensions)
             if micro_batch_index == self._micro_batch_per_rank - 1 and unit_index in self._open_windows:
                 self._optimizer.cpu_optimizer.close_window(self._open_windows.pop(unit_index))
-        else:
-            self._optimizer.cpu_optimizer.step(contexts, **extensions)
 
     # ---- statistics and decisions ---------------------------------------------------------------
     def _begin_iteration_statistics(self) -> None:
@@ -473,7 +486,7 @@ class FlexTrainOptsCoordinator:
         if self._offload:
             self._optimizer.cpu_optimizer.stream_wait()
             self._optimizer.cpu_optimizer.synchronize()
-        else:
+        if any(self._unit_resident):
             torch.cuda.current_stream().synchronize()
 
     # ---- state files ---------------------------------------------------------------------------
@@ -491,7 +504,7 @@ class FlexTrainOptsCoordinator:
         self.synchronize()
         paths = []
         for u in range(self._num_units):
-            blocks = self._unit_opts[u] if self._offload else [b.cpu() for b in self._unit_opts[u]]
+            blocks = [b.cpu() for b in self._unit_opts[u]] if self._unit_resident[u] else self._unit_opts[u]
             paths.append(write_unit_opts(directory, u, blocks, share=BACKWARD_SHARE, rank=rank,
                                          checkpoint_interval=checkpoint_interval, fsync=fsync))
         return paths
@@ -505,7 +518,7 @@ class FlexTrainOptsCoordinator:
             raise RuntimeError("units %s are being stepped on the GPU; load after clear_backward_pipeline()" % sorted(self._open_windows))
         self.synchronize()
         for u in range(self._num_units):
-            if self._offload:
+            if not self._unit_resident[u]:
                 read_unit_opts(directory, u, self._unit_opts[u], share=BACKWARD_SHARE, rank=rank,
                                checkpoint_interval=checkpoint_interval)
             else:

@@ -30,7 +30,14 @@ def test_half_parameters_on_gpu_and_host_pieces(cuda, oracle, offload, windows, 
     _run_backward_pipeline(cuda, oracle, offload, windows, half_layout)
 
 
-def _run_backward_pipeline(cuda, oracle, offload, windows, half_layout):
+@pytest.mark.parametrize("windows,resident", [("copy_back", 1), ("off", 2), ("auto", 4)])
+def test_some_units_resident_the_others_streamed(cuda, oracle, windows, resident):
+    """offload with resident_units: units 0..R-1 keep their master state in HBM, the others stream
+    from pinned host memory; the same results either way."""
+    _run_backward_pipeline(cuda, oracle, True, windows, "gpu", resident_units=resident)
+
+
+def _run_backward_pipeline(cuda, oracle, offload, windows, half_layout, resident_units=0):
     from flextrain_amd import FlexTrainAdam
     from flextrain_amd.coordinator import FlexTrainOptsCoordinator
     from flextrain_amd.memory import pinned_empty
@@ -73,9 +80,11 @@ def _run_backward_pipeline(cuda, oracle, offload, windows, half_layout):
     coord = FlexTrainOptsCoordinator()
     coord.initialize(opt, halves, micro_batches, offload=offload, device=cuda,
                      unit_windows={"auto": None, "off": False}.get(windows, True),
-                     window_write_through=windows == "write_through")
+                     window_write_through=windows == "write_through", resident_units=resident_units)
     assert coord._unit_windows == (offload and windows != "off")  # small shares: the automatic choice is windows
-    assert coord.unit_master_parameter(0).is_pinned() == offload
+    assert [coord.unit_master_parameter(u).is_pinned() for u in range(num_units)] == \
+        [offload and u >= resident_units for u in range(num_units)]
+    assert all(coord.unit_master_parameter(u).is_cuda for u in range(num_units) if not offload or u < resident_units)
 
     # oracle state, seeded the same way
     state = [(to_np(flat[u].float()).copy(), np.zeros(unit_numel, np.float32), np.zeros(unit_numel, np.float32))
