@@ -83,6 +83,19 @@ def test_step_statistics_and_accumulation_beyond_2_pow_32_elements(cuda, oracle)
     for name, t, want_first in (("p", p, pn), ("m", m, mn), ("v", v, vn), ("h", h, hn)):
         assert max_ulp_gpu(t[:PERIOD], want_first) == 0, name
         assert _every_period_equals_the_first(t), name
+
+    # a second step through the many-contexts launch: two contexts of one group, cut at an odd element
+    # beyond 2**31, the second one longer than 2**31 elements and ending beyond 2**32
+    from flextrain_amd.param_group import StepContext
+    cut = PERIOD * 2049 + 1
+    group = {"step": 8}
+    eng._step_many([StepContext(group, h[:cut], p[:cut], g[:cut], [m[:cut], v[:cut]]),
+                    StepContext(group, h[cut:], p[cut:], g[cut:], [m[cut:], v[cut:]])])
+    oracle.adam_step(pn, half_bits(pat["g"]), mn, vn, step=8, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
+                     weight_decay=HP["weight_decay"], g_dtype=CODE[torch.bfloat16], half_out=hn, half_dtype=CODE[torch.bfloat16])
+    for name, t, want_first in (("p", p, pn), ("m", m, mn), ("v", v, vn), ("h", h, hn)):
+        assert max_ulp_gpu(t[:PERIOD], want_first) == 0, name
+        assert _every_period_equals_the_first(t), name
     del h, m, v
 
     # accumulation into the (now updated) fp32 array, source cleared, statistics in the same pass
