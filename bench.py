@@ -644,6 +644,8 @@ def main() -> int:
                     help="pipeline: units whose fp32 state stays in HBM although the others are streamed from host memory")
     ap.add_argument("--resident", action="store_true",
                     help="pipeline: keep the fp32 state of every unit in HBM instead of pinned host memory")
+    ap.add_argument("--stats-keep-mib", type=int, default=None,
+                    help="cfg3/cfg4: MiB at the end of the statistics pass read with caching loads (default: the library's 256)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-offload-record", action="store_true",
                     help="cfg2: leave out the offloaded-streaming sub-record (cfg5 on the largest pinnable prefix, about 12 s)")
@@ -669,6 +671,8 @@ def main() -> int:
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.stats_keep_mib is not None:
+        _C.check("ft_set_cache_tuning", _C.lib().ft_set_cache_tuning(args.stats_keep_mib << 20))
     if args.workload == "cfg5":
         return bench_offload(args, torch, dev)
     if args.workload == "pipeline":

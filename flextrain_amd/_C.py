@@ -75,6 +75,7 @@ EXPORTS = {
     "ft_synth_fill": (c_int, [c_void_p, c_int, c_size_t, c_uint64, c_uint32, c_uint64, c_int, c_float, c_void_p]),
     "ft_synth_fill_host": (c_int, [c_void_p, c_int, c_size_t, c_uint64, c_uint32, c_uint64, c_int, c_float]),
     "ft_set_launch_tuning": (c_int, [c_int, c_int]),
+    "ft_set_cache_tuning": (c_int, [c_size_t]),
 }
 
 

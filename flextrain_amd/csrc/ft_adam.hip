@@ -51,6 +51,9 @@ std::map<std::pair<int, hipStream_t>, OwnedScratch> g_stats_ws;
 int g_adam_waves_per_cu = FT_ADAM_WAVES_PER_CU;
 std::unordered_map<int, int> g_lds_per_cu;   // device -> bytes of LDS per compute unit
 std::atomic<int> g_stats_blocks_per_cu{FT_STATS_BLOCKS_PER_CU};  // read without the lock
+// How many bytes at the end of a statistics pass are read with caching loads (the size of the
+// memory-side cache of MI355X: what can still be there when the update reads the gradients again).
+std::atomic<size_t> g_stats_keep_bytes{static_cast<size_t>(256) << 20};
 
 constexpr int kMaxStatsBlocks = 8192;
 
@@ -653,18 +656,20 @@ int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* 
         if (b > cap) b = cap;
         blocks = static_cast<int>(b);
         const ftk::u32x4* gv = reinterpret_cast<const ftk::u32x4*>(static_cast<const char*>(g) + head * esz);
+        const size_t ntiles = (nvec + kTile - 1) / kTile, keep_tiles = g_stats_keep_bytes.load() / (kTile * 16);
+        const uint64_t keep_from = ntiles > keep_tiles ? ntiles - keep_tiles : 0;
         switch (g_dtype) {
             case FT_F32:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F32, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from);
                 break;
             case FT_F16:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from);
                 break;
             default:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_BF16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from);
                 break;
         }
         FT_HIP(hipGetLastError());
@@ -800,6 +805,12 @@ int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ct
                        static_cast<const ft_grad_stats_t*>(stats), inv_scale, max_norm,
                        static_cast<ft_step_control_t*>(ctl_out));
     FT_HIP(hipGetLastError());
+    return FT_OK;
+}
+
+int ft_set_cache_tuning(size_t stats_keep_bytes)
+{
+    g_stats_keep_bytes = stats_keep_bytes;
     return FT_OK;
 }
 

@@ -438,9 +438,16 @@ __device__ __forceinline__ void block_stats_epilogue(double lane_sum, uint32_t b
 // off by 3e-6).
 constexpr int kStatsFlushTiles = 16;
 
+// The gradients are read again by the update that follows the decision, so what of them still fits
+// the memory-side cache afterwards is worth keeping there: tiles from `keep_from_tile` on (the last
+// ones this pass touches) are read with ordinary loads, everything before with streaming loads that
+// leave nothing behind. The update's own traffic is streaming, so the kept lines survive until it
+// reaches them. Measured on the 7B-layer partition (405 MB of fp16 gradients, 256 MB cache): the
+// update behind an all-streaming pass takes 0.838 ms, behind a caching pass 0.79 ms.
 template <int GT, int BLOCK, int UNROLL>
 __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restrict__ g, uint64_t nvec,
-                                                           float pre_mult, StatsPartial* __restrict__ partials)
+                                                           float pre_mult, StatsPartial* __restrict__ partials,
+                                                           uint64_t keep_from_tile)
 {
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     double lane_sum = 0.0;
@@ -452,8 +459,16 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
         const uint64_t base = tile * kTile + threadIdx.x;
         if ((tile + 1) * kTile <= nvec) {
             u32x4 w[UNROLL];
+            if (tile < keep_from_tile) {
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) w[u] = __builtin_nontemporal_load(g + base + (uint64_t)u * BLOCK);
+                for (int u = 0; u < UNROLL; ++u) w[u] = __builtin_nontemporal_load(g + base + (uint64_t)u * BLOCK);
+            } else {  // buffer loads with the default cache policy: a distinct instruction, so the two paths stay two
+                const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(g + tile * kTile), 0,
+                                                                                   (int)(kTile * 16), kRawBufferFlags);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+                    w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, 0);
+            }
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(w[u], pre_mult, acc, bad);
         } else {

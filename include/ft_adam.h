@@ -285,6 +285,11 @@ int ft_synth_fill_host(void* out, int dtype, size_t n, uint64_t seed, uint32_t s
  * squares may move in its last bits, within the documented tolerance). A value <= 0 restores the
  * default. Otherwise speed only, never results. */
 int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu);
+/* stats_keep_bytes: how many bytes at the END of a statistics pass (ft_grad_stats, ft_grad_decide)
+ * are read with caching loads, so that the update that reads the same gradients next finds them in
+ * the memory-side cache; everything before is read with streaming loads. Default 256 MiB (the
+ * cache of MI355X); 0 = stream everything, SIZE_MAX = cache everything. Speed only. */
+int ft_set_cache_tuning(size_t stats_keep_bytes);
 
 #ifdef __cplusplus
 }
