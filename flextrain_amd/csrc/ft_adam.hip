@@ -222,6 +222,27 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
 
     if (!vec_ok) return scalar_part(0, n);
 
+    // An in-place segment with edge elements is one launch of the many-segment kernel (tiles and
+    // edges in the same grid) instead of up to three.
+    const bool in_place = out.p == p && out.m == m && out.v == v;
+    if (in_place && (head > 0 || head + body < n) && ntiles + 1 < ftk::kMultiMaxWorkgroups) {
+        ftk::AdamMultiArgs ma;
+        ma.first_wg[0] = 0;
+        for (int k = 1; k < ftk::kMultiMaxSegments; ++k) ma.first_wg[k] = 0xffffffffu;
+        ma.ctl = ctl;
+        ftk::AdamSegment& d = ma.seg[0];
+        d.p = p;
+        d.g = g;
+        d.m = m;
+        d.v = v;
+        d.h = h;
+        d.n = n;
+        d.head = static_cast<uint32_t>(head);
+        d.body_tiles = static_cast<uint32_t>(ntiles);
+        d.c = c;
+        return launch_adam_multi(ma, GT, h != nullptr, HT, static_cast<unsigned>(ntiles) + 1u, stream);
+    }
+
     if (ntiles > 0) {
         ftk::AdamArgs a;
         a.p = p + head;
