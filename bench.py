@@ -454,9 +454,25 @@ def bench_pipeline_resident(args, torch, dev, Unit) -> int:
     from flextrain_amd.coordinator import FlexTrainOptsCoordinator
     n, mb, units = N_7B_LAYER, args.micro_batches, args.layers
     flat = [(torch.randn(n, device=dev) * 0.02).to(torch.bfloat16) for _ in range(units)]
-    params = [torch.nn.Parameter(f) for f in flat]
-    opt = FlexTrainAdam([{"params": params}], unit_parameter_map={u: Unit([params[u]]) for u in range(units)},
-                        aligned_unit_numel=n, offload=False, **{k: HP[k] for k in ("lr", "betas", "eps", "weight_decay")})
+    hp = {k: HP[k] for k in ("lr", "betas", "eps", "weight_decay")}
+    if args.layer_groups:
+        # A decoder layer as its own tensors in module order (input norm, q, k, v, o, post-attention
+        # norm, gate, up, down), matrices in a weight-decay group and the two norms in a group without:
+        # the group boundaries cut some shares into several step contexts.
+        h, f = 4096, 11008
+        sizes = [h, h * h, h * h, h * h, h * h, h, h * f, h * f, h * f]
+        decay, plain, unit_params = [], [], []
+        for fl in flat:
+            pieces = [torch.nn.Parameter(t) for t in fl.split(sizes)]
+            unit_params.append(pieces)
+            for t, size in zip(pieces, sizes):
+                (plain if size == h else decay).append(t)
+        groups = [{"params": decay}, {"params": plain, "weight_decay": 0.0}]
+    else:
+        unit_params = [[torch.nn.Parameter(fl)] for fl in flat]
+        groups = [{"params": [u[0] for u in unit_params]}]
+    opt = FlexTrainAdam(groups, unit_parameter_map={u: Unit(unit_params[u]) for u in range(units)},
+                        aligned_unit_numel=n, offload=False, **hp)
     coord = FlexTrainOptsCoordinator()
     coord.initialize(opt, flat, mb, offload=False)
     grads = (torch.randn(n, device=dev) * 1e-3).to(torch.bfloat16)
@@ -492,7 +508,8 @@ def bench_pipeline_resident(args, torch, dev, Unit) -> int:
         "data": "synthetic",
         "config": {"workload": f"pipeline, resident: coordinator schedule over {units} Llama-7B layers, {mb} shares per unit, "
                                "fp32 state, bf16 grads and parameters all in HBM",
-                   "elements": total, "units": units, "micro_batches": mb, "bytes_per_element": 34},
+                   "elements": total, "units": units, "micro_batches": mb, "bytes_per_element": 34,
+                   "contexts_per_unit": sum(len(coord._unit_step_ctxts[0][k]) for k in range(mb))},
         "host_ms_per_iteration": sum(host) / len(host) * 1e3,
         "roofline": {"bound": "hbm", "kernel": "adam_tile_kernel per share + gradient copy + clear", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None},
@@ -642,6 +659,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=32, help="cfg5: decoder layers (32 = the full 7B optimizer)")
     ap.add_argument("--resident-units", type=int, default=0,
                     help="pipeline: units whose fp32 state stays in HBM although the others are streamed from host memory")
+    ap.add_argument("--layer-groups", action="store_true",
+                    help="pipeline --resident: each layer as its nine tensors in two parameter groups (matrices with weight "
+                         "decay, norms without), so that group boundaries cut shares into several step contexts")
     ap.add_argument("--resident", action="store_true",
                     help="pipeline: keep the fp32 state of every unit in HBM instead of pinned host memory")
     ap.add_argument("--stats-keep-mib", type=int, default=None,
