@@ -163,7 +163,8 @@ int ft_grad_accumulate_decide(void* acc, int acc_dtype, void* g, int g_dtype, si
  * library runs on, held until the process ends), so the call allocates and frees nothing, whatever
  * the size of earlier calls. At most FT_STATIC_MAX_ELEMS elements per call (FT_EINVAL beyond).
  * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two
- * threads) race on it and must be ordered by the caller. */
+ * threads) race on it and must be ordered by the caller. The first call on a device looks the
+ * array's address up (hipGetSymbolAddress): make that call before a graph capture begins. */
 #define FT_STATIC_MAX_ELEMS (1ull << 28)
 int ft_grad_accumulate_static(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
                               float stats_pre_mult, void* stats_out, int stats_accumulate, void* stream);
