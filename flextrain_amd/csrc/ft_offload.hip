@@ -82,6 +82,13 @@ constexpr size_t kStagedMinElems = 32u * 1024u * 1024u;
 // one burst run at 49 GB/s each way, 290 chunks at 27-36 GB/s, whatever the host does about it.
 constexpr size_t kMaxChunksPerStep = 96;
 
+// A long step ramps in and out: its first and its last chunk's worth of elements go as quarter
+// chunks, so that the part of the pipeline that cannot overlap (the first copy in, the last copy
+// out) is a quarter of a chunk each instead of a whole one. That costs kRampExtraChunks more chunks
+// per step and is done for steps of at least kRampMinChunks chunks only.
+constexpr size_t kRampMinChunks = 8;
+constexpr size_t kRampExtraChunks = 6;
+
 struct Engine {
     uint32_t magic = 0x46544f45;  // "FTOE"
     std::mutex mu;                // one call at a time per handle; different handles are independent
@@ -541,9 +548,9 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     // array keeps its contents. (p, m and v need no such care: a skipped kernel whose outputs are
     // not its inputs copies the old state through.)
     const bool stage_h = half_out && half_on_host && out_staged && !ctl;
-    if ((in_staged || out_staged) && (n + e->chunk - 1) / e->chunk > kMaxChunksPerStep) {
-        const size_t mi = 1u << 20;
-        const size_t grown = ((n + kMaxChunksPerStep - 1) / kMaxChunksPerStep + mi - 1) / mi * mi;
+    if ((in_staged || out_staged) && (n + e->chunk - 1) / e->chunk + kRampExtraChunks > kMaxChunksPerStep) {
+        const size_t mi = 1u << 20, full = kMaxChunksPerStep - kRampExtraChunks;
+        const size_t grown = ((n + full - 1) / full + mi - 1) / mi * mi;
         if ((rc = resize_slots(e, grown)) != FT_OK) return rc;
     }
     if ((in_staged || out_staged) && !e->slots.back().v && (rc = resize_slots(e, e->chunk)) != FT_OK) return rc;
@@ -553,8 +560,23 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
         if (stage_h && !s.h) FT_HIP(hipMalloc(&s.h, chunk * 2));
     }
 
-    for (size_t off = 0; off < n; off += chunk) {
-        const size_t cnt = (n - off < chunk) ? (n - off) : chunk;
+    // Chunk sizes of this step. Every chunk but the last starts and ends on a multiple of 256
+    // elements (whole tiles at 1 KiB boundaries) whenever the chunk size itself is one.
+    const size_t quarter = (chunk / 4) & ~static_cast<size_t>(255);
+    const bool ramp = (in_staged || out_staged) && quarter > 0 && n / chunk >= kRampMinChunks;
+    std::vector<size_t> sizes;
+    if (ramp) {
+        const size_t body_end = (n - 4 * quarter) & ~static_cast<size_t>(255);
+        for (int k = 0; k < 4; ++k) sizes.push_back(quarter);
+        for (size_t off = 4 * quarter; off < body_end; off += chunk) sizes.push_back(body_end - off < chunk ? body_end - off : chunk);
+        for (int k = 0; k < 3; ++k) sizes.push_back(quarter);
+        sizes.push_back(n - body_end - 3 * quarter);
+    } else {
+        for (size_t off = 0; off < n; off += chunk) sizes.push_back(n - off < chunk ? n - off : chunk);
+    }
+    size_t off = 0;
+    for (size_t index = 0; index < sizes.size(); off += sizes[index], ++index) {
+        const size_t cnt = sizes[index];
         float *kp = hp + off, *km = hm + off, *kv = hv + off;          // kernel inputs
         float *op = hp + off, *om = hm + off, *ov = hv + off;          // kernel outputs
         const void* kg = gb + off * gsz;
