@@ -57,7 +57,7 @@ from typing import List, Optional, Sequence, Union
 import torch
 from torch import Tensor
 
-from .memory import RotateContainer, allocate_memory_chunks
+from .memory import RotateContainer, allocate_device_arrays, allocate_memory_chunks
 from .optimizer import FlexTrainOptimizer
 from .param_group import StepContextContainer
 
@@ -223,9 +223,11 @@ class FlexTrainOptsCoordinator:
 
         # [master | exp_avg | exp_avg_sq] per unit.
         per_element = 1 + optimizer.optimizer_state_per_element
+        # Resident units: the arrays of an update in one allocation with staggered starts (the layout
+        # the update kernel was never slow with); streamed units: exact-size pinned blocks.
         self._unit_opts = [
-            list(allocate_memory_chunks(self._unit_numel, per_element, master_dtype,
-                                        device if self._unit_resident[u] else torch.device("cpu")))
+            list(allocate_device_arrays([(self._unit_numel, master_dtype)] * per_element, device)) if self._unit_resident[u]
+            else list(allocate_memory_chunks(self._unit_numel, per_element, master_dtype, torch.device("cpu")))
             for u in range(self._num_units)]
 
         # Seed the master copy from the low-precision parameters (exact: widening conversion).
