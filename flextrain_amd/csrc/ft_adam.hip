@@ -443,6 +443,14 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
         // dynamic LDS so that the bytes in flight per compute unit stay at the tuned level.
         size_t waves = (nvec + 63) / 64;
         if (waves > 0x7fffffffu) waves = 0x7fffffffu;
+        // A pass that ends in a decision is followed by the update, which reads the accumulator as
+        // its gradients: the last stats_keep_bytes of it are stored with the default cache policy so
+        // that the update finds them in the memory-side cache (everything else streams).
+        uint64_t keep_from = ~0ull;
+        if (dec.ctl) {
+            const size_t tiles = (nvec + 63) / 64, keep_tiles = g_stats_keep_bytes.load() / (64 * 4 * asz);
+            keep_from = tiles > keep_tiles ? tiles - keep_tiles : 0;
+        }
         ftk::WavePartial* wave_parts =
             STATS ? reinterpret_cast<ftk::WavePartial*>(reinterpret_cast<char*>(parts) + ft_grad_stats_workspace_bytes())
                   : nullptr;
@@ -450,7 +458,7 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
                            fth::throttle_lds_bytes(4 * static_cast<unsigned>(asz + gsz)), stream,
                            static_cast<void*>(static_cast<char*>(acc) + head * asz),
                            static_cast<void*>(static_cast<char*>(g) + head * gsz), static_cast<uint64_t>(nvec), scale,
-                           pre_mult, wave_parts);
+                           pre_mult, wave_parts, keep_from);
         FT_HIP(hipGetLastError());
         if (STATS) {
             reduce_blocks = waves < static_cast<size_t>(kReduceBlocks) ? static_cast<int>(waves) : kReduceBlocks;

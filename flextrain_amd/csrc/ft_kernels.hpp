@@ -135,6 +135,17 @@ __device__ __forceinline__ void st_stream(__amdgpu_buffer_rsrc_t r, uint32_t byt
     __builtin_amdgcn_raw_buffer_store_b64(x, r, (int)byte_offset, 0, kAuxStreamStore);
 }
 
+// The same stores with the default cache policy: for the part of an array that its next reader
+// should find in the memory-side cache.
+__device__ __forceinline__ void st_keep(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, f32x4 x)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, x), r, (int)byte_offset, 0, 0);
+}
+__device__ __forceinline__ void st_keep(__amdgpu_buffer_rsrc_t r, uint32_t byte_offset, u32x2 x)
+{
+    __builtin_amdgcn_raw_buffer_store_b64(x, r, (int)byte_offset, 0, 0);
+}
+
 // Gradient unit = 4 consecutive elements.
 template <int GT, bool NT>
 __device__ __forceinline__ f32x4 load_g4(const void* g, uint64_t unit)
@@ -597,7 +608,7 @@ __device__ __forceinline__ void stats_of_stored(float value, uint32_t bits, floa
 // descriptors cover only the units of this tile that exist, so lanes past nvec cannot store.
 template <int AT, int GT, bool ZERO, bool STATS>
 __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t tile, uint64_t nvec, float scale,
-                                                float pre_mult, float (&sums)[4], uint32_t& bad)
+                                                float pre_mult, float (&sums)[4], uint32_t& bad, bool keep)
 {
     constexpr uint32_t kAccUnit = (AT == FT_F32) ? 16 : 8, kGradUnit = (GT == FT_F32) ? 16 : 8;
     const uint64_t t0 = tile * 64;  // wave-uniform
@@ -625,7 +636,10 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
         r[k] = x;
     }
     if constexpr (AT == FT_F32) {
-        st_stream(racc, threadIdx.x * kAccUnit, r);
+        if (keep)
+            st_keep(racc, threadIdx.x * kAccUnit, r);
+        else
+            st_stream(racc, threadIdx.x * kAccUnit, r);
         if constexpr (STATS) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -637,7 +651,10 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
         u32x2 w;
         w.x = pack2<AT>(r.x, r.y);
         w.y = pack2<AT>(r.z, r.w);
-        st_stream(racc, threadIdx.x * kAccUnit, w);
+        if (keep)
+            st_keep(racc, threadIdx.x * kAccUnit, w);
+        else
+            st_stream(racc, threadIdx.x * kAccUnit, w);
         if constexpr (STATS) {
             const uint32_t b[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
 #pragma unroll
@@ -666,13 +683,14 @@ struct WavePartial {
 // the grid had to be capped). With STATS every workgroup writes wave_partials[blockIdx.x].
 template <int AT, int GT, bool ZERO, bool STATS>
 __global__ __launch_bounds__(64) void grad_accumulate_kernel(void* acc, void* g, uint64_t nvec, float scale,
-                                                             float pre_mult, WavePartial* __restrict__ wave_partials)
+                                                             float pre_mult, WavePartial* __restrict__ wave_partials,
+                                                             uint64_t keep_from_tile)
 {
     float sums[4] = {0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
     const uint64_t ntiles = (nvec + 63) / 64;
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x)
-        accumulate_tile<AT, GT, ZERO, STATS>(acc, g, tile, nvec, scale, pre_mult, sums, bad);
+        accumulate_tile<AT, GT, ZERO, STATS>(acc, g, tile, nvec, scale, pre_mult, sums, bad, tile >= keep_from_tile);
     if constexpr (STATS) {
         const float t = wave_sum((sums[0] + sums[1]) + (sums[2] + sums[3]));
         const uint32_t tb = wave_sum_u32(bad);

@@ -216,13 +216,20 @@ class GradientGuard:
         return target
 
     def accumulate(self, acc: torch.Tensor, grads: torch.Tensor, scale: float = 1.0, zero_grads: bool = False,
-                   with_stats: bool = False, loss_scale: float = 1.0) -> None:
+                   with_stats: bool = False, loss_scale: float = 1.0, decide: bool = False,
+                   max_grad_norm: Optional[float] = None) -> Optional[torch.Tensor]:
         """``acc += scale * grads`` in one pass (one fused multiply-add per element, rounded to
         ``acc``'s dtype), optionally clearing ``grads`` and -- ``with_stats`` -- gathering the
         statistics of the new ``acc`` as ``add(acc, loss_scale)`` would, so that the last
         accumulation of a step needs no separate statistics pass. Replaces the reference's
         per-micro-batch ``gradacc_buffer += extra_grads`` and ``zero_`` pair
-        (``flextrain/memory/coordinator/optimizer.py:743,775-777``)."""
+        (``flextrain/memory/coordinator/optimizer.py:743,775-777``).
+
+        ``decide`` (implies ``with_stats``): the pass also takes the step decision from the record as
+        it then stands, like ``decide_async``, and returns the control record -- for the last
+        accumulation before an update of the same buffer. The tail of ``acc`` is then left in the
+        memory-side cache for that update to find."""
+        with_stats = with_stats or decide
         for name, t in (("acc", acc), ("grads", grads)):
             if not t.is_cuda or not t.is_contiguous():
                 raise ValueError(f"{name} must be a contiguous GPU tensor")
@@ -234,13 +241,22 @@ class GradientGuard:
             if need > self._ws_bytes:  # grows with the largest buffer seen (8 bytes per 256 elements)
                 self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
                 self._ws_bytes = need
+        inv_scale = float(1.0 / float(loss_scale))
         with torch.cuda.device(acc.device):
-            _C.check("ft_grad_accumulate", self._lib.ft_grad_accumulate(
-                acc.data_ptr(), _C.dtype_code(acc.dtype), grads.data_ptr(), _C.dtype_code(grads.dtype), acc.numel(),
-                float(scale), int(bool(zero_grads)), float(1.0 / float(loss_scale)), stats_ptr,
-                0 if self._fresh else 1, self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(acc.device)))
+            if decide:
+                _C.check("ft_grad_accumulate_decide", self._lib.ft_grad_accumulate_decide(
+                    acc.data_ptr(), _C.dtype_code(acc.dtype), grads.data_ptr(), _C.dtype_code(grads.dtype), acc.numel(),
+                    float(scale), int(bool(zero_grads)), inv_scale, stats_ptr, 0 if self._fresh else 1, inv_scale,
+                    float(max_grad_norm) if max_grad_norm else 0.0, self.control.data_ptr(), self._ws.data_ptr(),
+                    self._ws_bytes, _C.current_stream_ptr(acc.device)))
+            else:
+                _C.check("ft_grad_accumulate", self._lib.ft_grad_accumulate(
+                    acc.data_ptr(), _C.dtype_code(acc.dtype), grads.data_ptr(), _C.dtype_code(grads.dtype), acc.numel(),
+                    float(scale), int(bool(zero_grads)), inv_scale, stats_ptr,
+                    0 if self._fresh else 1, self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(acc.device)))
         if with_stats:
             self._fresh = False
+        return self.control if decide else None
 
     def decide_async(self, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None,
                      out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import CODE, NORM_RTOL, max_ulp_gpu, to_np
+from _util import CODE, NORM_RTOL, half_bits, max_ulp_gpu, to_np
 
 pytestmark = pytest.mark.gpu
 
@@ -95,3 +95,33 @@ def test_accumulate_llama7b_layer(cuda, oracle):
     bad, sumsq = oracle.grad_stats(an, CODE[torch.float32])
     assert d.nonfinite == bad == 0
     assert abs(math.sqrt(d.sumsq) - math.sqrt(sumsq)) <= NORM_RTOL * math.sqrt(sumsq)
+
+
+def test_accumulate_with_decision_in_one_call(cuda, oracle):
+    """GradientGuard.accumulate(decide=True): accumulate + statistics + decision, then the update of
+    the same buffer under that decision (the accumulator's tail is stored with caching stores for
+    it); against the oracle, with a clip below 1."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.loss_scaler import GradientGuard
+    n = 3_000_017
+    gen = torch.Generator(device=cuda).manual_seed(77)
+    acc = torch.randn(n, device=cuda, generator=gen) * 0.01
+    g = (torch.randn(n, device=cuda, generator=gen) * 0.02 * 32).to(torch.float16)
+    p = torch.randn(n, device=cuda, generator=gen) * 0.02
+    m, v = torch.zeros(n, device=cuda), torch.zeros(n, device=cuda)
+    p0 = to_np(p).copy()
+    accn = to_np(acc).copy()
+    oracle.grad_accumulate(accn, CODE[torch.float32], half_bits(g).copy(), CODE[torch.float16], scale=0.5)
+    guard = GradientGuard(cuda)
+    guard.begin()
+    ctl = guard.accumulate(acc, g, scale=0.5, decide=True, loss_scale=32.0, max_grad_norm=1.0)
+    eng = FlexTrainCPUAdam(lr=1e-3, weight_decay=0.01)
+    eng._step({"step": 1}, None, p, acc, m, v, control=ctl)
+    d = guard.read()
+    assert np.array_equal(to_np(acc).view(np.uint32), accn.view(np.uint32))
+    bad, sumsq = oracle.grad_stats(accn, CODE[torch.float32], pre_mult=1.0 / 32)
+    assert d.nonfinite == bad == 0 and abs(d.sumsq - sumsq) <= 2e-6 * sumsq and d.clip_coef < 1.0
+    pn, mn, vn = p0, np.zeros(n, np.float32), np.zeros(n, np.float32)
+    oracle.adam_step(pn, accn, mn, vn, step=1, lr=1e-3, weight_decay=0.01, grad_mult=d.grad_mult)
+    assert np.array_equal(to_np(p).view(np.uint32), pn.view(np.uint32))
+    assert np.array_equal(to_np(m).view(np.uint32), mn.view(np.uint32)) and np.array_equal(to_np(v).view(np.uint32), vn.view(np.uint32))
