@@ -25,6 +25,7 @@ class AdamSegment(ctypes.Structure):
         ("n", c_size_t), ("step", c_uint64),
         ("lr", c_float), ("beta1", c_float), ("beta2", c_float), ("eps", c_float), ("weight_decay", c_float),
         ("bias_correction", ctypes.c_int32), ("grad_mult", c_float), ("reserved", ctypes.c_int32),
+        ("hyper", c_void_p),
     ]
 
 
@@ -44,6 +45,9 @@ EXPORTS = {
     "ft_adam_step": (c_int, [c_int, c_uint64, c_float, c_float, c_float, c_float, c_float, c_int, c_float,
                              c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_size_t,
                              c_void_p, c_void_p]),
+    "ft_adam_hyper_fill": (c_int, [c_int, c_uint64, c_float, c_float, c_float, c_float, c_float, c_int, c_float, c_void_p]),
+    "ft_adam_step_hyper": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_size_t,
+                                   c_void_p, c_void_p]),
     "ft_adam_step_multi": (c_int, [c_int, POINTER(AdamSegment), c_int, c_int, c_int, c_void_p, c_void_p]),
     "ft_grad_stats_workspace_bytes": (c_size_t, []),
     "ft_grad_stats": (c_int, [c_void_p, c_int, c_size_t, c_float, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
@@ -52,6 +56,8 @@ EXPORTS = {
                                    c_void_p, c_size_t, c_void_p]),
     "ft_grad_decide": (c_int, [c_void_p, c_int, c_size_t, c_float, c_void_p, c_int, c_float, c_float, c_void_p, c_void_p, c_size_t,
                                c_void_p]),
+    "ft_grad_decide_dev": (c_int, [c_void_p, c_int, c_size_t, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_size_t,
+                                   c_void_p]),
     "ft_grad_accumulate_decide": (c_int, [c_void_p, c_int, c_void_p, c_int, c_size_t, c_float, c_int, c_float, c_void_p, c_int,
                                           c_float, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ft_grad_accumulate_static": (c_int, [c_void_p, c_int, c_void_p, c_int, c_size_t, c_float, c_int, c_float, c_void_p, c_int,

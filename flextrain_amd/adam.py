@@ -32,6 +32,46 @@ DEFAULT_OFFLOAD_CHUNK = 64 * 1024 * 1024
 DEFAULT_OFFLOAD_SLOTS = 3
 
 
+#: key under which a parameter group carries its device-resident scalars (``make_capturable``)
+HYPER_KEY = "hyper_record"
+
+
+class HyperRecord:
+    """The per-step scalars of one parameter group (step count folded into the bias corrections,
+    learning rate, betas, epsilon, weight decay) in device memory, with a pinned host staging copy.
+
+    By default those scalars reach the kernels by value, so a HIP graph that records a step replays
+    the step count and learning rate of the moment it was recorded. A group that carries a record
+    has them read from device memory instead: ``fill()`` computes them on the host exactly as the
+    by-value path does and writes the pinned staging copy (call it whenever ``group["step"]`` or a
+    hyper-parameter changes; outside any capture; it waits for the device first, so that a step still
+    in flight reads the values it was enqueued with); ``sync()`` enqueues the 48-byte copy to the device
+    on the current stream -- recorded into a graph, that copy re-reads the staging copy at every
+    replay, so a recorded step follows the group from iteration to iteration."""
+
+    def __init__(self, engine: "FlexTrainCPUAdam", device: torch.device):
+        self._engine = engine
+        self.host = torch.zeros(12, dtype=torch.int32, pin_memory=True)
+        self.dev = torch.zeros(12, dtype=torch.int32, device=device)
+
+    def fill(self, group_args: Dict, grad_mult: float = 1.0) -> "HyperRecord":
+        assert STEP_KEY in group_args, f"Key '{STEP_KEY}' not found in parameter group arguments."
+        # A step enqueued earlier (or a graph replay) may not have copied the staging values yet:
+        # they may only change once that work is done.
+        torch.cuda.synchronize(self.dev.device)
+        self._engine._set_defaults_args(group_args)
+        beta1, beta2 = group_args["betas"]
+        _C.check("ft_adam_hyper_fill", self._engine._lib.ft_adam_hyper_fill(
+            self._engine.opt_id, int(group_args[STEP_KEY]), float(group_args["lr"]), float(beta1), float(beta2),
+            float(group_args["eps"]), float(group_args["weight_decay"]), int(bool(group_args["bias_correction"])),
+            float(grad_mult), self.host.data_ptr()))
+        return self
+
+    def sync(self) -> "HyperRecord":
+        self.dev.copy_(self.host, non_blocking=True)
+        return self
+
+
 def _flat(name: str, t: Tensor, dtype_ok, numel: int) -> Tensor:
     if t.dtype not in dtype_ok:
         raise ValueError(f"{name} has dtype {t.dtype}, expected one of {sorted(map(str, dtype_ok))}")
@@ -174,11 +214,21 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
                     if name == "half_parameter" and not t.is_cuda and t.is_pinned():
                         continue  # the kernel writes the copy into pinned host memory over the link
                     raise ValueError(f"{name} is on {t.device} but full_parameter is on {full_parameter.device}")
+            record = group_args.get(HYPER_KEY)
             with torch.cuda.device(full_parameter.device):
-                _C.check("ft_adam_step", self._lib.ft_adam_step(
-                    self.opt_id, *hyper, full_parameter.data_ptr(), gradient.data_ptr(), g_code,
-                    exp_avg.data_ptr(), exp_avg_sq.data_ptr(), h_ptr, h_code, n, ctl_ptr,
-                    _C.current_stream_ptr(full_parameter.device)))
+                if record is not None:  # the scalars are read from device memory (see HyperRecord)
+                    if grad_mult != 1.0:
+                        raise ValueError("a group with device-resident scalars takes its multiplier from the record "
+                                         "(HyperRecord.fill(group, grad_mult=...)) or from a control record")
+                    _C.check("ft_adam_step_hyper", self._lib.ft_adam_step_hyper(
+                        self.opt_id, record.dev.data_ptr(), full_parameter.data_ptr(), gradient.data_ptr(), g_code,
+                        exp_avg.data_ptr(), exp_avg_sq.data_ptr(), h_ptr, h_code, n, ctl_ptr,
+                        _C.current_stream_ptr(full_parameter.device)))
+                else:
+                    _C.check("ft_adam_step", self._lib.ft_adam_step(
+                        self.opt_id, *hyper, full_parameter.data_ptr(), gradient.data_ptr(), g_code,
+                        exp_avg.data_ptr(), exp_avg_sq.data_ptr(), h_ptr, h_code, n, ctl_ptr,
+                        _C.current_stream_ptr(full_parameter.device)))
             return
 
         # offloaded: master state in pinned host memory
@@ -248,10 +298,28 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             seg.beta1, seg.beta2 = group["betas"]
             seg.eps, seg.weight_decay = float(group["eps"]), float(group["weight_decay"])
             seg.bias_correction, seg.grad_mult = int(bool(group["bias_correction"])), float(grad_mult)
+            record = group.get(HYPER_KEY)
+            if record is not None:
+                if grad_mult != 1.0:
+                    raise ValueError("a group with device-resident scalars takes its multiplier from the record or a control record")
+                seg.hyper = record.dev.data_ptr()
         with torch.cuda.device(device):
             _C.check("ft_adam_step_multi", self._lib.ft_adam_step_multi(
                 self.opt_id, segs, len(live), _C.dtype_code(g_dtype), _C.dtype_code(half_dtype), ctl_ptr,
                 _C.current_stream_ptr(device)))
+
+    def make_capturable(self, group_args: Dict, device=None) -> HyperRecord:
+        """Gives the parameter group a ``HyperRecord`` (kept under ``group_args["hyper_record"]``) and
+        fills it from the group's present values: resident steps of that group then read their scalars
+        from device memory and may be recorded into a HIP graph once and replayed across iterations.
+        The caller keeps the record current: ``record.fill(group)`` after changing ``step`` or a
+        hyper-parameter, ``record.sync()`` in front of the step (inside the recorded region)."""
+        device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
+        record = group_args.get(HYPER_KEY)
+        if record is None:
+            group_args.setdefault(STEP_KEY, 0)
+            record = group_args[HYPER_KEY] = HyperRecord(self, device)
+        return record.fill(group_args)
 
     def open_window(self, full_parameter: Tensor, exp_avg: Tensor, exp_avg_sq: Tensor, write_through: bool = False) -> int:
         """Brings the whole master state of one unit (three pinned host tensors of equal length) to

@@ -8,6 +8,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <string.h>
 
 #include <atomic>
 #include <cmath>
@@ -177,7 +178,7 @@ struct OutPtrs {
 
 template <int GT, int HT>
 int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, float* v, void* h, size_t n,
-                 const ft_step_control_t* ctl, hipStream_t stream, OutPtrs out)
+                 const ft_step_control_t* ctl, hipStream_t stream, OutPtrs out, const ftk::AdamConsts* hyper)
 {
     constexpr size_t gsz = (GT == FT_F32) ? 4 : 2;
     const char* gb = reinterpret_cast<const char*>(g);
@@ -209,6 +210,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.v_out = out.v + off;
         a.h = h ? hb + off * 2 : nullptr;
         a.ctl = ctl;
+        a.hyper = hyper;
         a.n = cnt;
         a.c = c;
         size_t blocks = (cnt + 255) / 256;
@@ -239,6 +241,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         d.n = n;
         d.head = static_cast<uint32_t>(head);
         d.body_tiles = static_cast<uint32_t>(ntiles);
+        d.hyper = hyper;
         d.c = c;
         return launch_adam_multi(ma, GT, h != nullptr, HT, static_cast<unsigned>(ntiles) + 1u, stream);
     }
@@ -254,6 +257,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.v_out = out.v + head;
         a.h = h ? hb + head * 2 : nullptr;
         a.ctl = ctl;
+        a.hyper = hyper;
         a.n = ntiles * ftk::kWave;
         a.c = c;
         const unsigned lds = throttle_lds_bytes(48 + 4 * static_cast<unsigned>(gsz));
@@ -276,18 +280,18 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
 
 template <int GT>
 int launch_g(const ftk::AdamConsts& c, float* p, const void* g, float* m, float* v, void* h, int half_dtype,
-             size_t n, const ft_step_control_t* ctl, hipStream_t stream, OutPtrs out)
+             size_t n, const ft_step_control_t* ctl, hipStream_t stream, OutPtrs out, const ftk::AdamConsts* hyper)
 {
-    if (h == nullptr) return launch_typed<GT, -1>(c, p, g, m, v, nullptr, n, ctl, stream, out);
-    if (half_dtype == FT_F16) return launch_typed<GT, FT_F16>(c, p, g, m, v, h, n, ctl, stream, out);
-    return launch_typed<GT, FT_BF16>(c, p, g, m, v, h, n, ctl, stream, out);
+    if (h == nullptr) return launch_typed<GT, -1>(c, p, g, m, v, nullptr, n, ctl, stream, out, hyper);
+    if (half_dtype == FT_F16) return launch_typed<GT, FT_F16>(c, p, g, m, v, h, n, ctl, stream, out, hyper);
+    return launch_typed<GT, FT_BF16>(c, p, g, m, v, h, n, ctl, stream, out, hyper);
 }
 
 }  // namespace
 
 int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, float* m, float* v,
                 void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream,
-                float* p_out, float* m_out, float* v_out)
+                float* p_out, float* m_out, float* v_out, const ftk::AdamConsts* hyper)
 {
     if (n == 0) return FT_OK;
     if (!p || !g || !m || !v) return fail(FT_EINVAL, "params, grads, exp_avg and exp_avg_sq must not be NULL");
@@ -298,13 +302,14 @@ int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, 
         (half_out && !aligned(half_out, 2)))
         return fail(FT_EALIGN, "a pointer is not aligned to its element size");
     if (ctl && !aligned(ctl, 16)) return fail(FT_EALIGN, "ft_step_control_t must be 16-byte aligned");
+    if (hyper && !aligned(hyper, 16)) return fail(FT_EALIGN, "ft_adam_hyper_t must be 16-byte aligned");
     const OutPtrs out{p_out ? p_out : p, m_out ? m_out : m, v_out ? v_out : v};
     if (!aligned(out.p, 4) || !aligned(out.m, 4) || !aligned(out.v, 4))
         return fail(FT_EALIGN, "an output pointer is not aligned to its element size");
     switch (g_dtype) {
-        case FT_F32: return launch_g<FT_F32>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out);
-        case FT_F16: return launch_g<FT_F16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out);
-        default: return launch_g<FT_BF16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out);
+        case FT_F32: return launch_g<FT_F32>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out, hyper);
+        case FT_F16: return launch_g<FT_F16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out, hyper);
+        default: return launch_g<FT_BF16>(c, p, g, m, v, half_out, half_dtype, n, ctl, stream, out, hyper);
     }
 }
 
@@ -396,6 +401,7 @@ struct Decide {
     float inv_scale = 1.0f;
     float max_norm = 0.0f;
     ft_step_control_t* ctl = nullptr;
+    const float* scale_dev = nullptr;  // 1/loss_scale in device memory: replaces pre_mult and inv_scale
 };
 
 // Statistics scratch of ft_grad_accumulate_static: block partials followed by one wavefront partial
@@ -507,7 +513,7 @@ extern "C" {
 
 const char* ft_last_error(void) { return t_last_error.c_str(); }
 
-int ft_abi_version(void) { return 1; }
+int ft_abi_version(void) { return 2; }
 
 int ft_device_count(void)
 {
@@ -558,6 +564,34 @@ int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, floa
                             static_cast<hipStream_t>(stream));
 }
 
+int ft_adam_hyper_fill(int id, uint64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
+                       int bias_correction, float grad_mult, ft_adam_hyper_t* out)
+{
+    static_assert(sizeof(ftk::AdamConsts) <= sizeof(ft_adam_hyper_t), "the public record must hold the kernels' scalars");
+    if (!out) return fth::fail(FT_EINVAL, "out must not be NULL");
+    fth::AdamObject o;
+    int rc = fth::find_adam(id, &o);
+    if (rc != FT_OK) return rc;
+    const ftk::AdamConsts c =
+        fth::make_consts(step, lr, beta1, beta2, eps, weight_decay, bias_correction != 0, o.adamw_mode, grad_mult);
+    memset(out, 0, sizeof *out);
+    memcpy(out, &c, sizeof c);
+    return FT_OK;
+}
+
+int ft_adam_step_hyper(int id, const void* hyper_dev, void* p, const void* g, int g_dtype, void* m, void* v, void* half_out,
+                       int half_dtype, size_t n, const void* ctl, void* stream)
+{
+    fth::AdamObject o;
+    int rc = fth::find_adam(id, &o);
+    if (rc != FT_OK) return rc;
+    if (!hyper_dev) return fth::fail(FT_EINVAL, "hyper_dev must not be NULL");
+    ftk::AdamConsts unused{};  // every scalar comes from the device record
+    return fth::launch_adam(unused, static_cast<float*>(p), g, g_dtype, static_cast<float*>(m), static_cast<float*>(v), half_out,
+                            half_dtype, n, static_cast<const ft_step_control_t*>(ctl), static_cast<hipStream_t>(stream), nullptr,
+                            nullptr, nullptr, static_cast<const ftk::AdamConsts*>(hyper_dev));
+}
+
 int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_dtype, int half_dtype,
                        const void* ctl_, void* stream_)
 {
@@ -581,6 +615,7 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
         if (!aligned(sg.p, 4) || !aligned(sg.m, 4) || !aligned(sg.v, 4) || !aligned(sg.g, gsz) ||
             (sg.half_out && !aligned(sg.half_out, 2)))
             return fth::fail(FT_EALIGN, "segment %d: a pointer is not aligned to its element size", i);
+        if (sg.hyper && !aligned(sg.hyper, 16)) return fth::fail(FT_EALIGN, "segment %d: ft_adam_hyper_t must be 16-byte aligned", i);
     }
     // Two batches fill side by side (with and without a low-precision copy: two kernel variants);
     // a batch is launched when it holds kMultiMaxSegments segments or its grid is full.
@@ -618,7 +653,8 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
             // arrays whose alignments disagree (element by element), or a segment too long for one
             // grid: the single-segment path takes it
             rc = fth::launch_adam(c, p, sg.g, g_dtype, static_cast<float*>(sg.m), static_cast<float*>(sg.v), sg.half_out,
-                                  half_dtype, sg.n, ctl, stream);
+                                  half_dtype, sg.n, ctl, stream, nullptr, nullptr, nullptr,
+                                  static_cast<const ftk::AdamConsts*>(sg.hyper));
             if (rc != FT_OK) return rc;
             continue;
         }
@@ -636,6 +672,7 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
         d.n = sg.n;
         d.head = static_cast<uint32_t>(head);
         d.body_tiles = static_cast<uint32_t>(body_tiles);
+        d.hyper = static_cast<const ftk::AdamConsts*>(sg.hyper);
         d.c = c;
         b.a.first_wg[b.count] = (b.workgroups << 4) | static_cast<unsigned>(b.count);
         b.workgroups += wgs;
@@ -690,15 +727,15 @@ int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* 
         switch (g_dtype) {
             case FT_F32:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F32, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev);
                 break;
             case FT_F16:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev);
                 break;
             default:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_BF16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev);
                 break;
         }
         FT_HIP(hipGetLastError());
@@ -707,15 +744,15 @@ int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* 
     switch (g_dtype) {
         case FT_F32:
             hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl);
+                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl, dec.scale_dev);
             break;
         case FT_F16:
             hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl);
+                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl, dec.scale_dev);
             break;
         default:
             hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_BF16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl);
+                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl, dec.scale_dev);
             break;
     }
     FT_HIP(hipGetLastError());
@@ -742,6 +779,19 @@ int ft_grad_decide(const void* g, int g_dtype, size_t n, float pre_mult, void* s
     dec.max_norm = max_norm;
     dec.ctl = static_cast<ft_step_control_t*>(ctl_out);
     return grad_stats_impl(g, g_dtype, n, pre_mult, stats, accumulate, workspace, workspace_bytes, dec, stream);
+}
+
+int ft_grad_decide_dev(const void* g, int g_dtype, size_t n, const void* inv_scale_dev, void* stats, int accumulate,
+                       float max_norm, void* ctl_out, void* workspace, size_t workspace_bytes, void* stream)
+{
+    if (!ctl_out || !inv_scale_dev) return fth::fail(FT_EINVAL, "ctl_out and inv_scale_dev must not be NULL");
+    if (!aligned(ctl_out, 16)) return fth::fail(FT_EALIGN, "ft_step_control_t must be 16-byte aligned");
+    if (!aligned(inv_scale_dev, 4)) return fth::fail(FT_EALIGN, "inv_scale_dev must be 4-byte aligned");
+    Decide dec;
+    dec.max_norm = max_norm;
+    dec.ctl = static_cast<ft_step_control_t*>(ctl_out);
+    dec.scale_dev = static_cast<const float*>(inv_scale_dev);
+    return grad_stats_impl(g, g_dtype, n, 1.0f, stats, accumulate, workspace, workspace_bytes, dec, stream);
 }
 
 }  // extern "C"

@@ -38,7 +38,8 @@ ftk::AdamConsts make_consts(uint64_t step, float lr, float beta1, float beta2, f
 // p_out/m_out/v_out: where the new values are written; nullptr = in place.
 int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, float* m, float* v,
                 void* half_out, int half_dtype, size_t n, const ft_step_control_t* ctl, hipStream_t stream,
-                float* p_out = nullptr, float* m_out = nullptr, float* v_out = nullptr);
+                float* p_out = nullptr, float* m_out = nullptr, float* v_out = nullptr,
+                const ftk::AdamConsts* hyper = nullptr);  // hyper: the scalars in device memory (they replace c)
 
 // Elements of a segment that go in front of its vector body (see the definition).
 size_t segment_head(const void* p, size_t n);

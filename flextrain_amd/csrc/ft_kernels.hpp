@@ -178,6 +178,12 @@ template <int GT, int HT, bool HAS_CTL>
 __global__ __launch_bounds__(kWave) void adam_tile_kernel(AdamArgs a, uint64_t tile0)
 {
     AdamConsts c = a.c;
+    // The by-value scalars are pinned in scalar registers here, so that their loads go out with the
+    // other kernel arguments and are not sunk behind the test of a.hyper (a second, dependent
+    // round of scalar loads in front of every tile's vector loads).
+    asm volatile("" : "+s"(c.beta1), "+s"(c.beta2), "+s"(c.omb1), "+s"(c.omb2), "+s"(c.bias2), "+s"(c.eps), "+s"(c.step_size),
+                 "+s"(c.wd_coef), "+s"(c.grad_mult), "+s"(c.wd_mode));
+    if (a.hyper) c = *a.hyper;  // the step's scalars kept in device memory (wave-uniform loads)
     const uint64_t t0 = (tile0 + blockIdx.x) * kWave;  // first unit of the tile: wave-uniform
     const uint64_t i = t0 + threadIdx.x;
     if constexpr (HAS_CTL) {  // wave-uniform scalar loads: one decision per step
@@ -221,6 +227,7 @@ template <int GT, int HT>
 __global__ __launch_bounds__(256) void adam_scalar_kernel(AdamArgs a)
 {
     AdamConsts c = a.c;
+    if (a.hyper) c = *a.hyper;
     const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
     if (a.ctl) {
         if (a.ctl->skip) {  // out of place: the old state still has to reach the outputs
@@ -293,6 +300,7 @@ __global__ __launch_bounds__(kWave) void adam_multi_kernel(AdamMultiArgs a)
     c.wd_coef = sg->c.wd_coef;
     c.grad_mult = sg->c.grad_mult;
     c.wd_mode = sg->c.wd_mode;
+    if (const AdamConsts* hyper = sg->hyper) c = *hyper;  // the segment's scalars kept in device memory
     if constexpr (HAS_CTL) {
         if (a.ctl->skip) return;
         c.grad_mult = a.ctl->grad_mult;
@@ -458,8 +466,9 @@ constexpr int kStatsFlushTiles = 16;
 template <int GT, int BLOCK, int UNROLL>
 __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restrict__ g, uint64_t nvec,
                                                            float pre_mult, StatsPartial* __restrict__ partials,
-                                                           uint64_t keep_from_tile)
+                                                           uint64_t keep_from_tile, const float* scale_dev)
 {
+    if (scale_dev) pre_mult = *scale_dev;  // 1/loss_scale kept in device memory (wave-uniform load)
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     double lane_sum = 0.0;
     uint32_t bad = 0;
@@ -539,8 +548,10 @@ __global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartia
                                                                int nparts, const void* g, uint64_t head,
                                                                uint64_t tail_begin, uint64_t n, float pre_mult,
                                                                ft_grad_stats_t* out, int accumulate, float inv_scale,
-                                                               float max_norm, ft_step_control_t* ctl)
+                                                               float max_norm, ft_step_control_t* ctl,
+                                                               const float* scale_dev)
 {
+    if (scale_dev) pre_mult = inv_scale = *scale_dev;
     __shared__ double s_sum[256];
     __shared__ uint64_t s_bad[256];
     double s = 0.0;

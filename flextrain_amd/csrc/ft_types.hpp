@@ -26,6 +26,7 @@ struct AdamArgs {
     float* v_out;
     void* h;                       // low-precision copy or nullptr
     const ft_step_control_t* ctl;  // device decision or nullptr
+    const AdamConsts* hyper;       // the scalars in device memory (they replace c), or nullptr
     uint64_t n;                    // elements (scalar kernel) or 4-element units (vector kernel)
     AdamConsts c;
 };
@@ -44,6 +45,7 @@ struct AdamSegment {
     uint64_t n;           // elements
     uint32_t head;        // elements in front of the first tile (they reach the alignment the tiles want)
     uint32_t body_tiles;  // whole 256-element tiles behind the head
+    const AdamConsts* hyper;  // the scalars in device memory (they replace c), or nullptr
     AdamConsts c;
 };
 

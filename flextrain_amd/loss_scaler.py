@@ -165,9 +165,18 @@ class GradientGuard:
     control buffer to hand to ``_step(control=...)``).
     """
 
-    def __init__(self, device=None):
+    def __init__(self, device=None, capturable: bool = False):
+        """``capturable``: 1/loss_scale is read by the kernels from device memory instead of travelling
+        by value, so that a step recorded into a HIP graph follows a loss scale that changes between
+        replays: ``set_scale()`` writes a pinned staging copy (outside any capture), and
+        ``add_and_decide`` first enqueues the 4-byte copy to the device (recorded, it re-reads the
+        staging copy at every replay)."""
         self.device = torch.device(device) if device is not None else torch.device("cuda", torch.cuda.current_device())
         self._lib = _C.lib()
+        self.capturable = bool(capturable)
+        if self.capturable:
+            self._scale_host = torch.ones(1, dtype=torch.float32, pin_memory=True)
+            self._scale_dev = torch.ones(1, dtype=torch.float32, device=self.device)
         # 32 bytes: ft_grad_stats_t followed by ft_step_control_t, read back with one copy
         self._buf = torch.zeros(4, dtype=torch.float64, device=self.device)
         self._ws_bytes = int(self._lib.ft_grad_stats_workspace_bytes())
@@ -196,6 +205,11 @@ class GradientGuard:
                 0 if self._fresh else 1, self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(grads.device)))
         self._fresh = False
 
+    def set_scale(self, loss_scale: float) -> None:
+        """Capturable guards: the loss scale the next (recorded or eager) ``add_and_decide`` works with."""
+        torch.cuda.synchronize(self.device)  # a step in flight still reads the present value
+        self._scale_host[0] = float(1.0 / float(loss_scale))
+
     def add_and_decide(self, grads: torch.Tensor, loss_scale: float = 1.0, max_grad_norm: Optional[float] = None,
                        out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``add(grads)`` followed by ``decide_async(...)`` with one launch fewer: the kernel that
@@ -208,10 +222,17 @@ class GradientGuard:
             raise ValueError("out must be 16 bytes of 16-byte aligned device memory")
         inv_scale = float(1.0 / float(loss_scale))
         with torch.cuda.device(grads.device):
-            _C.check("ft_grad_decide", self._lib.ft_grad_decide(
-                grads.data_ptr(), _C.dtype_code(grads.dtype), grads.numel(), inv_scale, self.stats_ptr,
-                0 if self._fresh else 1, inv_scale, float(max_grad_norm) if max_grad_norm else 0.0, target.data_ptr(),
-                self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(grads.device)))
+            if self.capturable:  # the scale comes from device memory; `loss_scale` is not used (see set_scale)
+                self._scale_dev.copy_(self._scale_host, non_blocking=True)
+                _C.check("ft_grad_decide_dev", self._lib.ft_grad_decide_dev(
+                    grads.data_ptr(), _C.dtype_code(grads.dtype), grads.numel(), self._scale_dev.data_ptr(), self.stats_ptr,
+                    0 if self._fresh else 1, float(max_grad_norm) if max_grad_norm else 0.0, target.data_ptr(),
+                    self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(grads.device)))
+            else:
+                _C.check("ft_grad_decide", self._lib.ft_grad_decide(
+                    grads.data_ptr(), _C.dtype_code(grads.dtype), grads.numel(), inv_scale, self.stats_ptr,
+                    0 if self._fresh else 1, inv_scale, float(max_grad_norm) if max_grad_norm else 0.0, target.data_ptr(),
+                    self._ws.data_ptr(), self._ws_bytes, _C.current_stream_ptr(grads.device)))
         self._fresh = False
         return target
 

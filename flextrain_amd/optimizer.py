@@ -185,6 +185,10 @@ class FlexTrainOptimizer:
         max_grad_norm: clip the global L2 norm of the unscaled gradients to this value.
         grad_reduce_fn: called with the flat gradient buffer before anything else (the place of
             the reference's ``all_reduce(AVG)``, ``:250``); default none (one GPU).
+        capturable: keep every group's per-step scalars (and 1/loss_scale) in device memory, so that
+            ``enqueue_step()`` can be recorded into a HIP graph once and replayed every iteration:
+            ``update_states()`` refreshes the pinned staging copies, the recorded region copies them
+            to the device. Resident state only.
     """
 
     cpu_optimizer: FlexTrainCPUOptimizer = None
@@ -202,6 +206,7 @@ class FlexTrainOptimizer:
         loss_scaler=None,
         max_grad_norm: Optional[float] = None,
         grad_reduce_fn: Optional[Callable[[Tensor], None]] = None,
+        capturable: bool = False,
     ):
         assert isinstance(param_groups, Iterable)
         assert self.cpu_optimizer is not None, "a subclass must create self.cpu_optimizer first"
@@ -305,6 +310,12 @@ class FlexTrainOptimizer:
         )
         self.last_step_skipped = False
         self.last_grad_norm: Optional[float] = None
+        self.capturable = bool(capturable)
+        if self.capturable:
+            if self._offload:
+                raise ValueError("capturable=True needs resident state (offload=False): the streamed step blocks on the host")
+            for group in self.param_groups:
+                self.cpu_optimizer.make_capturable(group, device)
 
     @property
     def optimizer_state_per_element(self) -> int:
@@ -339,17 +350,26 @@ class FlexTrainOptimizer:
             self._grad_reduce_fn(grads)
         extensions = {}
         self._step_guarded = (self.loss_scaler is not None or self.max_grad_norm is not None) and grads.numel() > 0
+        if self.capturable:
+            for group in self.param_groups:  # 48-byte copies; recorded, they re-read the staging copies at every replay
+                group["hyper_record"].sync()
         if self._step_guarded:
-            from .loss_scaler import GradientGuard  # local import: keeps module load light
-            if not hasattr(self, "_guard"):
-                self._guard = GradientGuard(device=grads.device)
             scale = float(self.loss_scaler.loss_scale) if self.loss_scaler is not None else 1.0
+            self._step_guard(grads.device)
             self._guard.begin()
             extensions["control"] = self._guard.add_and_decide(grads, loss_scale=scale, max_grad_norm=self.max_grad_norm)
         self.cpu_optimizer.step(self.non_layerwise_step_contexts, **extensions)
         self._zero_grads()
         if self._offload and self._device_dtype == self._master_dtype:
             self._device_para.copy_(self._master_para, non_blocking=True)
+
+    def _step_guard(self, device):
+        if not hasattr(self, "_guard"):
+            from .loss_scaler import GradientGuard  # local import: keeps module load light
+            self._guard = GradientGuard(device=device, capturable=self.capturable)
+            if self.capturable:
+                self._guard.set_scale(float(self.loss_scaler.loss_scale) if self.loss_scaler is not None else 1.0)
+        return self._guard
 
     def complete_step(self) -> bool:
         """Host side of a step, after ``enqueue_step()`` (or after replaying a graph that holds it):
@@ -362,6 +382,8 @@ class FlexTrainOptimizer:
         self.last_grad_norm = decision.grad_norm
         if self.loss_scaler is not None:
             self.loss_scaler.update_scale(decision.overflow)
+            if self.capturable:  # what the next (replayed) step unscales with
+                self._guard.set_scale(float(self.loss_scaler.loss_scale))
         self.last_step_skipped = bool(decision.overflow)
         return not decision.overflow
 
@@ -374,3 +396,5 @@ class FlexTrainOptimizer:
         """Advances ``group["step"]`` of every group (reference ``:265-272``)."""
         for group in self.param_groups:
             group[STEP_KEY] = group.get(STEP_KEY, 0) + 1
+            if self.capturable:  # staging copy only: the step itself brings it to the device
+                group["hyper_record"].fill(group)

@@ -87,6 +87,22 @@ int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, floa
                  int g_dtype, void* m, void* v, void* half_out, int half_dtype, size_t n,
                  const void* ctl, void* stream);
 
+/* ---- the step's scalars in device memory ----------------------------------------------------
+ * ft_adam_step passes step, lr, the bias corrections ... to the kernel by value, as the reference
+ * does per call (cpu_adam_impl.cpp:212-295); a HIP graph that records such a launch replays those
+ * values. For callers that record the step once and replay it every iteration, the scalars can
+ * live in device memory instead: ft_adam_hyper_fill computes the record on the HOST exactly as
+ * ft_adam_step would (cpu_adam.h:67-102,148-166), the caller copies its 48 bytes to device memory
+ * (a copy recorded in the graph re-reads the host staging at every replay), and ft_adam_step_hyper /
+ * ft_adam_segment_t.hyper make the kernel read it from there. Same results as by value. */
+typedef struct ft_adam_hyper_t {
+    uint32_t words[12]; /* opaque */
+} ft_adam_hyper_t;
+int ft_adam_hyper_fill(int id, uint64_t step, float lr, float beta1, float beta2, float eps, float weight_decay,
+                       int bias_correction, float grad_mult, ft_adam_hyper_t* host_out);
+int ft_adam_step_hyper(int id, const void* hyper_dev, void* p, const void* g, int g_dtype, void* m, void* v, void* half_out,
+                       int half_dtype, size_t n, const void* ctl, void* stream);
+
 /* ---- many resident updates in one launch -------------------------------------------------------
  * Replaces the loop of flextrain/optimizer.py:44-69 (one adam_update[_copy] call per StepContext;
  * flextrain/param_group.py:365-477 cuts a unit's share into one context per parameter group and
@@ -109,6 +125,7 @@ typedef struct ft_adam_segment_t {
     int32_t bias_correction;
     float grad_mult;
     int32_t reserved;   /* 0 */
+    const void* hyper;  /* NULL, or a device ft_adam_hyper_t: it replaces step ... grad_mult above */
 } ft_adam_segment_t;
 int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_dtype, int half_dtype,
                        const void* ctl, void* stream);
@@ -155,6 +172,11 @@ int ft_grad_decide(const void* g, int g_dtype, size_t n, float pre_mult, void* s
 int ft_grad_accumulate_decide(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
                               float stats_pre_mult, void* stats, int stats_accumulate, float inv_scale, float max_norm,
                               void* ctl_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ft_grad_decide_dev: ft_grad_decide with 1/loss_scale read from device memory (one float, used both
+ * as pre_mult and as inv_scale), for a recorded step whose loss scale changes between replays. */
+int ft_grad_decide_dev(const void* g, int g_dtype, size_t n, const void* inv_scale_dev, void* stats, int accumulate,
+                       float max_norm, void* ctl_out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ft_grad_accumulate_static: ft_grad_accumulate for callers that cannot allocate (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc). No counterpart in the

@@ -242,6 +242,48 @@ void many_segments_one_launch(hipStream_t stream)
     }
     check(same_bits(dp, p) && same_bits(dm, m) && same_bits(dv, v) && same_bits(dh, h),
           "many segments: every segment bit-identical to the CPU checker, nothing outside them touched");
+    // the same step with every scalar read from device memory: a second copy of the state must end up identical
+    {
+        std::vector<float> p2(p), m2(m), v2(v);  // the state after the first step: step it once more, both ways
+        std::vector<uint16_t> h2(h);
+        float *ep = dev_copy(p2), *em = dev_copy(m2), *ev = dev_copy(v2);
+        uint16_t* eh = dev_copy(h2);
+        ft_adam_hyper_t host_rec[3];
+        ft_adam_hyper_t* dev_rec = nullptr;
+        HIP_OK(hipMalloc(reinterpret_cast<void**>(&dev_rec), sizeof host_rec));
+        ft_adam_segment_t by_value[3], by_record[3];
+        for (int k = 0; k < 3; ++k) {
+            FT_OK_OR_DIE(ft_adam_hyper_fill(9, step[k] + 1, lr[k], B1, B2, EPS, wd[k], 1, 0.5f, &host_rec[k]));
+            by_value[k] = segs[k];
+            by_value[k].step = step[k] + 1;
+            by_value[k].grad_mult = 0.5f;
+            by_record[k] = segs[k];
+            by_record[k].p = ep + lo[k];
+            by_record[k].m = em + lo[k];
+            by_record[k].v = ev + lo[k];
+            by_record[k].half_out = eh + lo[k];
+            by_record[k].step = 999;       // ignored: the record decides
+            by_record[k].lr = 123.f;
+            by_record[k].hyper = dev_rec + k;
+        }
+        HIP_OK(hipMemcpyAsync(dev_rec, host_rec, sizeof host_rec, hipMemcpyHostToDevice, stream));
+        FT_OK_OR_DIE(ft_adam_step_multi(9, by_value, 3, FT_BF16, FT_BF16, nullptr, stream));
+        FT_OK_OR_DIE(ft_adam_step_multi(9, by_record, 2, FT_BF16, FT_BF16, nullptr, stream));
+        FT_OK_OR_DIE(ft_adam_step_hyper(9, dev_rec + 2, ep + lo[2], dg + lo[2], FT_BF16, em + lo[2], ev + lo[2], eh + lo[2], FT_BF16, len[2],
+                                        nullptr, stream));
+        HIP_OK(hipStreamSynchronize(stream));
+        HIP_OK(hipMemcpy(p2.data(), dp, total * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(m2.data(), dm, total * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(v2.data(), dv, total * 4, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(h2.data(), dh, total * 2, hipMemcpyDeviceToHost));
+        check(same_bits(ep, p2) && same_bits(em, m2) && same_bits(ev, v2) && same_bits(eh, h2),
+              "scalars from device memory: the same bits as by value (many segments and single call)");
+        HIP_OK(hipMemcpy(dp, p.data(), total * 4, hipMemcpyHostToDevice));  // back to the state the checks below expect
+        HIP_OK(hipMemcpy(dm, m.data(), total * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dv, v.data(), total * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dh, h.data(), total * 2, hipMemcpyHostToDevice));
+        HIP_OK(hipFree(ep)); HIP_OK(hipFree(em)); HIP_OK(hipFree(ev)); HIP_OK(hipFree(eh)); HIP_OK(hipFree(dev_rec));
+    }
     segs[1].m = nullptr;
     check(ft_adam_step_multi(9, segs, 3, FT_BF16, FT_BF16, nullptr, stream) == FT_EINVAL, "many segments: a NULL array is refused");
     HIP_OK(hipStreamSynchronize(stream));

@@ -224,3 +224,72 @@ def test_non_layerwise_step_replays_in_a_hip_graph(cuda):
         for se, sr in zip(eager.non_layerwise_step_contexts[0].optimizer_states, replayed.non_layerwise_step_contexts[0].optimizer_states):
             assert torch.equal(se, sr), replay
         assert not replayed._device_grad.any()
+
+
+def test_capturable_step_follows_step_count_learning_rate_and_loss_scale_across_replays(cuda):
+    """FlexTrainOptimizer(capturable=True): the groups' scalars and 1/loss_scale live in device
+    memory, so ONE recorded enqueue_step() is replayed over real iterations -- the step count
+    advances, the learning rate follows a schedule, the dynamic loss scale halves after an overflow --
+    and stays bit-equal to a twin optimizer stepped eagerly with by-value scalars."""
+    from flextrain_amd import FlexTrainAdam
+    from flextrain_amd.loss_scaler import DynamicLossScaler
+
+    def build(capturable):
+        torch.manual_seed(8)
+        a = torch.nn.Parameter((torch.randn(257, 300, device=cuda) * 0.02).to(torch.float16))
+        b = torch.nn.Parameter((torch.randn(4099, device=cuda) * 0.02).to(torch.float16))
+        groups = [{"params": [a], "weight_decay": 0.1}, {"params": [b], "weight_decay": 0.0, "lr": 3e-4}]
+        opt = FlexTrainAdam(groups, lr=1e-3, loss_scaler=DynamicLossScaler(init_scale=2048.0, delayed_shift=1, scale_window=3),
+                            max_grad_norm=1.0, capturable=capturable)
+        return opt, groups, (a, b)
+
+    eager, eager_groups, eager_params = build(False)
+    replayed, replay_groups, replay_params = build(True)
+    gen = torch.Generator(device=cuda).manual_seed(9)
+
+    def fresh_gradients(overflow):
+        scale = eager.loss_scaler.loss_scale
+        assert replayed.loss_scaler.loss_scale == scale
+        for pe, pr in zip(eager_params, replay_params):
+            g = (torch.randn(pe.shape, device=cuda, generator=gen) * 0.3 * scale).to(torch.float16)
+            if overflow and pe.dim() == 1:
+                g[5] = float("inf")
+            pe.grad.copy_(g)
+            pr.grad.copy_(g)
+
+    def advance(iteration):
+        for groups, opt in ((eager_groups, eager), (replay_groups, replayed)):
+            groups[0]["lr"] = 1e-3 * (0.9 ** iteration)  # a schedule, changed before update_states refreshes the records
+            opt.update_states()
+
+    advance(0)
+    fresh_gradients(False)
+    assert eager.step() is True and replayed.step() is True  # warm-up, eagerly
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    advance(1)
+    fresh_gradients(False)
+    with torch.cuda.graph(graph, stream=side):
+        replayed.enqueue_step()
+    torch.cuda.synchronize()
+    seen_scales = []
+    for iteration, overflow in enumerate([False, True, False, False, False, True, False], start=1):
+        if iteration > 1:
+            advance(iteration)
+            fresh_gradients(overflow)
+        seen_scales.append(eager.loss_scaler.loss_scale)
+        torch.cuda.synchronize()
+        graph.replay()
+        assert replayed.complete_step() is (not overflow)
+        assert eager.step() is (not overflow)
+        torch.cuda.synchronize()
+        assert torch.equal(replayed._master_para, eager._master_para), iteration
+        assert torch.equal(replayed._device_para, eager._device_para), iteration
+        for ce, cr in zip(eager.non_layerwise_step_contexts, replayed.non_layerwise_step_contexts):
+            for se, sr in zip(ce.optimizer_states, cr.optimizer_states):
+                assert torch.equal(se, sr), iteration
+        assert replayed.loss_scaler.loss_scale == eager.loss_scaler.loss_scale
+    moves = [b - a for a, b in zip(seen_scales, seen_scales[1:]) if b != a]
+    assert any(d < 0 for d in moves) and any(d > 0 for d in moves)  # the scale fell and rose between replays
+    assert replay_groups[0]["step"] == 8

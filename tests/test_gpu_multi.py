@@ -250,4 +250,4 @@ def test_bad_segments_are_refused_before_anything_runs(cuda):
     assert lib.ft_adam_step_multi(eng.opt_id, None, 0, _C.F32, _C.F16, None, stream) == 0
     torch.cuda.synchronize()
     assert torch.equal(P, before), "a refused call must not have stepped its first segment"
-    assert ctypes.sizeof(_C.AdamSegment) == 88
+    assert ctypes.sizeof(_C.AdamSegment) == 96
