@@ -79,8 +79,13 @@ int ft_adam_destroy(int id);
  *               round-to-nearest-even bfloat16
  *   ctl         NULL, or a device ft_step_control_t read by the kernel: it overrides
  *               grad_mult and can turn the whole call into a no-op (skip)
- * p, m, v: fp32, n elements, updated in place. Pointers must be aligned to their element size;
- * full speed needs p/m/v 16-byte and 16-bit arrays 8-byte aligned at the same element offset.
+ * p, m, v: fp32, n elements, updated in place. Pointers must be aligned to their element size.
+ * The vector path needs every array to reach its vector alignment (16 bytes; 8 for the 16-bit
+ * arrays) after the same number of elements, which views cut at a common element offset of aligned
+ * flat buffers (the reference's StepContext views) always do; the call then steps the elements in
+ * front of the first 1 KiB boundary of p and behind the last whole 256-element tile separately
+ * (same launch for an in-place update) so that every tile covers whole cache lines. Arrays whose
+ * alignments disagree are stepped element by element: correct, about 1.5x slower.
  */
 int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, float eps,
                  float weight_decay, int bias_correction, float grad_mult, void* p, const void* g,
@@ -166,7 +171,9 @@ int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n,
 /* ft_grad_decide / ft_grad_accumulate_decide: ft_grad_stats / ft_grad_accumulate (with statistics)
  * followed by ft_grad_control on the record as it then stands, without the extra launch: the last
  * kernel of the statistics pass writes the decision too. For the pass that completes a step's
- * statistics (the last gradient buffer, the last micro-batch). Same results as the two calls. */
+ * statistics (the last gradient buffer, the last micro-batch). Same results as the two calls.
+ * Both leave the end of what the update will read next (the last stats_keep_bytes of g, of acc: see
+ * ft_set_cache_tuning) in the memory-side cache. */
 int ft_grad_decide(const void* g, int g_dtype, size_t n, float pre_mult, void* stats, int accumulate, float inv_scale,
                    float max_norm, void* ctl_out, void* workspace, size_t workspace_bytes, void* stream);
 int ft_grad_accumulate_decide(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
