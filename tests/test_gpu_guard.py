@@ -109,11 +109,15 @@ def _check_state(tag, p, m, v, h, pn, mn, vn, hn):
     assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst["h"] <= HALF_ULP, (tag, worst)
 
 
-def test_config3_overflow_skips_and_scale_trace(cuda, oracle):
+@pytest.mark.parametrize("path", ["host_decision", "device_decision"])
+def test_config3_overflow_skips_and_scale_trace(cuda, oracle, path):
     """7B-layer partition, fp16 grads = N(0,1e-3) x loss scale, 8 steps, inf/nan injected at three
     seeded positions on steps 3 and 6: exactly those steps are skipped (state bit-identical), the
     scale goes 65536 -> 32768 -> 16384 (hysteresis 1), t advances only on applied steps, and every
-    applied step equals AdamW on the unscaled gradients."""
+    applied step equals AdamW on the unscaled gradients. Two ways through: the decision read back
+    before the update is launched, and -- as bench.py and the optimizer front ends run it -- statistics
+    and decision in one fused pass, the update launched blind under the device-side record, the
+    record read afterwards."""
     from flextrain_amd import FlexTrainCPUAdam
     from flextrain_amd.loss_scaler import DynamicLossScaler, GradientGuard
     n = N_7B_LAYER
@@ -138,21 +142,36 @@ def test_config3_overflow_skips_and_scale_trace(cuda, oracle):
             for k, kind in zip(rng.choice(n, size=3, replace=False), (float("inf"), float("-inf"), float("nan"))):
                 g[int(k)] = kind
         guard.begin()
-        guard.add(g, loss_scale=scale)
-        d = guard.decide(loss_scale=scale)
-        scaler.update_scale(d.overflow)
-        if d.overflow:
-            skipped.append(it)
-            before = [t.clone() for t in (p, m, v, h)]
-            # even if a caller launches the update with the device-side decision, nothing moves
-            eng._step({"step": group["step"] + 1}, h, p, g, m, v, control=guard.control)
-            for now, was in zip((p, m, v, h), before):
-                assert torch.equal(now, was)
-            assert d.nonfinite == 3
-            continue
-        group["step"] += 1
-        assert d.grad_mult == 1.0 / scale  # power of two: exact
-        eng._step(group, h, p, g, m, v, grad_mult=d.grad_mult)
+        if path == "device_decision":
+            before = [t.clone() for t in (p, m, v, h)] if it in (3, 6) else None
+            ctl = guard.add_and_decide(g, loss_scale=scale)
+            eng._step({"step": group["step"] + 1}, h, p, g, m, v, control=ctl)  # launched without knowing the decision
+            d = guard.read()
+            scaler.update_scale(d.overflow)
+            if d.overflow:
+                skipped.append(it)
+                for now, was in zip((p, m, v, h), before):
+                    assert torch.equal(now, was)
+                assert d.nonfinite == 3
+                continue
+            group["step"] += 1
+            assert d.grad_mult == 1.0 / scale
+        else:
+            guard.add(g, loss_scale=scale)
+            d = guard.decide(loss_scale=scale)
+            scaler.update_scale(d.overflow)
+            if d.overflow:
+                skipped.append(it)
+                before = [t.clone() for t in (p, m, v, h)]
+                # even if a caller launches the update with the device-side decision, nothing moves
+                eng._step({"step": group["step"] + 1}, h, p, g, m, v, control=guard.control)
+                for now, was in zip((p, m, v, h), before):
+                    assert torch.equal(now, was)
+                assert d.nonfinite == 3
+                continue
+            group["step"] += 1
+            assert d.grad_mult == 1.0 / scale  # power of two: exact
+            eng._step(group, h, p, g, m, v, grad_mult=d.grad_mult)
         hn = _apply_oracle(oracle, pn, mn, vn, g, group["step"], d.grad_mult, torch.bfloat16)
         if it in (1, 4, 8):
             _check_state(f"cfg3 it={it} t={group['step']}", p, m, v, h, pn, mn, vn, hn)
