@@ -474,21 +474,55 @@ def bench_pipeline_resident(args, torch, dev, Unit) -> int:
     opt = FlexTrainAdam(groups, unit_parameter_map={u: Unit(unit_params[u]) for u in range(units)},
                         aligned_unit_numel=n, offload=False, **hp)
     coord = FlexTrainOptsCoordinator()
-    coord.initialize(opt, flat, mb, offload=False)
+    coord.initialize(opt, flat, mb, offload=False, resident_shares=args.resident_shares or None,
+                     step_stream={"auto": None, "on": True, "off": False}[args.step_stream])
     grads = (torch.randn(n, device=dev) * 1e-3).to(torch.bfloat16)
     share = n // mb
 
-    def iteration():
+    # Optional stand-in for the arithmetic of a backward pass: per micro-batch, for each of the layer's
+    # seven matrices (a x b), one (T x a)(a x b) and one (a x T)(T x b) product in bf16 = 4 T a b flops,
+    # 4 x parameters x T in all, which is what the backward of a decoder layer over T tokens costs.
+    tokens = args.backward_tokens
+    if tokens:
+        shapes = [(4096, 4096)] * 4 + [(4096, 11008)] * 3
+        wide = {b: torch.randn(tokens, b, device=dev, dtype=torch.bfloat16) for b in (4096, 11008)}
+        x_t = torch.randn(4096, tokens, device=dev, dtype=torch.bfloat16)
+        x = torch.randn(tokens, 4096, device=dev, dtype=torch.bfloat16)
+        weights = {b: torch.randn(4096, b, device=dev, dtype=torch.bfloat16) for b in (4096, 11008)}
+        out_tb = {b: torch.empty(tokens, b, device=dev, dtype=torch.bfloat16) for b in (4096, 11008)}
+        out_ab = {b: torch.empty(4096, b, device=dev, dtype=torch.bfloat16) for b in (4096, 11008)}
+
+    def backward_arithmetic():
+        if tokens:
+            for _, b in shapes:
+                torch.mm(x, weights[b], out=out_tb[b])
+                torch.mm(x_t, wide[b], out=out_ab[b])
+
+    def iteration(with_optimizer=True):
+        if not with_optimizer:
+            for _ in range(units * mb):
+                backward_arithmetic()
+            return
         opt.update_states()
         for u in reversed(range(units)):
             buf = coord.pre_unit_backward(u)
             for k in range(mb):
+                backward_arithmetic()
                 buf[k * share:(k + 1) * share].copy_(grads[k * share:(k + 1) * share])
                 coord.post_micro_batch_backward(u, k)
         coord.clear_backward_pipeline()
 
     for _ in range(args.warmup):
         iteration()
+    arithmetic_ms = None
+    if tokens:
+        iteration(with_optimizer=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            iteration(with_optimizer=False)
+        torch.cuda.synchronize()
+        arithmetic_ms = (time.perf_counter() - t0) / args.steps * 1e3
     walls, host = [], []
     for _ in range(args.steps):
         torch.cuda.synchronize()
@@ -509,8 +543,11 @@ def bench_pipeline_resident(args, torch, dev, Unit) -> int:
         "config": {"workload": f"pipeline, resident: coordinator schedule over {units} Llama-7B layers, {mb} shares per unit, "
                                "fp32 state, bf16 grads and parameters all in HBM",
                    "elements": total, "units": units, "micro_batches": mb, "bytes_per_element": 34,
-                   "contexts_per_unit": sum(len(coord._unit_step_ctxts[0][k]) for k in range(mb))},
+                   "shares_per_unit": len(coord._unit_step_ctxts[0]),
+                   "contexts_per_unit": sum(len(coord._unit_step_ctxts[0][k]) for k in range(len(coord._unit_step_ctxts[0]))),
+                   "step_stream": coord._step_stream is not None, "backward_tokens": tokens},
         "host_ms_per_iteration": sum(host) / len(host) * 1e3,
+        **({"backward_arithmetic_ms": arithmetic_ms, "exposed_optimizer_ms": sec * 1e3 - arithmetic_ms} if tokens else {}),
         "roofline": {"bound": "hbm", "kernel": "adam_tile_kernel per share + gradient copy + clear", "achieved": achieved,
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": None},
     }), flush=True)
@@ -662,6 +699,13 @@ def main() -> int:
     ap.add_argument("--layer-groups", action="store_true",
                     help="pipeline --resident: each layer as its nine tensors in two parameter groups (matrices with weight "
                          "decay, norms without), so that group boundaries cut shares into several step contexts")
+    ap.add_argument("--resident-shares", type=int, default=0,
+                    help="pipeline --resident: launches a resident unit's update is cut into (0 = the coordinator's default)")
+    ap.add_argument("--step-stream", default="auto", choices=["auto", "on", "off"],
+                    help="pipeline --resident: updates on the coordinator's own stream beside the caller's kernels")
+    ap.add_argument("--backward-tokens", type=int, default=0,
+                    help="pipeline --resident: also run, per micro-batch, bf16 matrix products costing a decoder layer's "
+                         "backward pass over this many tokens (0 = only the gradient copy)")
     ap.add_argument("--resident", action="store_true",
                     help="pipeline: keep the fp32 state of every unit in HBM instead of pinned host memory")
     ap.add_argument("--stats-keep-mib", type=int, default=None,

@@ -15,6 +15,34 @@ class _Unit:
         self.paras = paras
 
 
+# How units whose state is in HBM are stepped: the default (the caller's stream, one launch per unit),
+# the reference's shape (one share per micro-batch), and either on the coordinator's own stream.
+RESIDENT_MODES = {
+    "caller_stream_one_share": {},
+    "own_stream_share_per_micro_batch": dict(step_stream=True, resident_shares="micro_batches"),
+    "caller_stream_share_per_micro_batch": dict(resident_shares="micro_batches"),
+    "own_stream_one_share": dict(step_stream=True),
+    "caller_stream_two_shares": dict(resident_shares=2),
+}
+
+
+def _with_resident_modes(cases):
+    """Every case in the default mode; the cases with all state in HBM also with one share per
+    micro-batch on the coordinator's own stream."""
+    out = []
+    for case in cases:
+        for mode in list(RESIDENT_MODES)[:1 if case[0] else 2]:
+            out.append(pytest.param(*case, mode, id="-".join(map(str, case)) + "-" + mode))
+    return out
+
+
+def _resident_kwargs(mode, micro_batches):
+    kwargs = dict(RESIDENT_MODES[mode])
+    if kwargs.get("resident_shares") == "micro_batches":
+        kwargs["resident_shares"] = micro_batches
+    return kwargs
+
+
 @pytest.mark.parametrize("offload,windows", [(True, "copy_back"), (True, "write_through"), (True, "off"), (True, "auto"), (False, "off")])
 def test_backward_pipeline_matches_oracle(cuda, oracle, offload, windows):
     _run_backward_pipeline(cuda, oracle, offload, windows, "gpu")
@@ -37,12 +65,29 @@ def test_some_units_resident_the_others_streamed(cuda, oracle, windows, resident
     _run_backward_pipeline(cuda, oracle, True, windows, "gpu", resident_units=resident)
 
 
-def _run_backward_pipeline(cuda, oracle, offload, windows, half_layout, resident_units=0):
+@pytest.mark.parametrize("mode", list(RESIDENT_MODES)[1:])
+@pytest.mark.parametrize("offload,resident", [(False, 0), (True, 2)])
+def test_resident_units_on_either_stream_in_any_number_of_shares(cuda, oracle, offload, resident, mode):
+    """A resident unit's update in one launch or one share per micro-batch, on the coordinator's own
+    stream or on the caller's: the same bits (the other tests run the default, the caller's stream
+    and one share). Low-precision parameters cut at an odd element."""
+    _run_backward_pipeline(cuda, oracle, offload, "copy_back", "split_odd", resident_units=resident, mode=mode)
+
+
+def test_step_stream_is_ordered_with_the_gradient_buffers(cuda, oracle):
+    """Units long enough (16 Mi elements) that an update on the coordinator's stream is still running
+    when the caller's stream is given the next unit's work: the buffer it reads must not be cleared
+    or refilled under it, and the record it is skipped by must be complete."""
+    _run_backward_pipeline(cuda, oracle, False, "off", "gpu", mode="own_stream_one_share", unit_numel=1 << 24, num_units=3)
+
+
+def _run_backward_pipeline(cuda, oracle, offload, windows, half_layout, resident_units=0, mode="caller_stream_one_share",
+                           unit_numel=1 << 20, num_units=4):
     from flextrain_amd import FlexTrainAdam
     from flextrain_amd.coordinator import FlexTrainOptsCoordinator
     from flextrain_amd.memory import pinned_empty
     torch.manual_seed(0)
-    num_units, micro_batches, unit_numel = 4, 4, 1 << 20
+    micro_batches = 4
     real = unit_numel - 4097  # the tail of each unit is alignment padding
     # each unit: a weight (decay) and a bias (no decay); the boundary falls inside a share
     w_numel, b_numel = real - 5000, 5000
@@ -80,7 +125,9 @@ def _run_backward_pipeline(cuda, oracle, offload, windows, half_layout, resident
     coord = FlexTrainOptsCoordinator()
     coord.initialize(opt, halves, micro_batches, offload=offload, device=cuda,
                      unit_windows={"auto": None, "off": False}.get(windows, True),
-                     window_write_through=windows == "write_through", resident_units=resident_units)
+                     window_write_through=windows == "write_through", resident_units=resident_units,
+                     **_resident_kwargs(mode, micro_batches))
+    assert (coord._step_stream is not None) == RESIDENT_MODES[mode].get("step_stream", False)
     assert coord._unit_windows == (offload and windows != "off")  # small shares: the automatic choice is windows
     assert [coord.unit_master_parameter(u).is_pinned() for u in range(num_units)] == \
         [offload and u >= resident_units for u in range(num_units)]
@@ -242,9 +289,9 @@ def _check_units(tag, coord, flat, state, expected_half):
         assert max(worst["p"], worst["m"], worst["v"]) <= MASTER_ULP and worst["h"] <= HALF_ULP, (tag, u, worst)
 
 
-@pytest.mark.parametrize("offload,windows,gradacc", [(False, False, None), (True, True, None), (True, False, None),
-                                                     (False, False, torch.float32), (True, True, torch.float32)])
-def test_scaled_gradients_and_overflow_while_stepping_during_backward(cuda, oracle, offload, windows, gradacc):
+@pytest.mark.parametrize("offload,windows,gradacc,mode", _with_resident_modes([
+    (False, False, None), (True, True, None), (True, False, None), (False, False, torch.float32), (True, True, torch.float32)]))
+def test_scaled_gradients_and_overflow_while_stepping_during_backward(cuda, oracle, offload, windows, gradacc, mode):
     """fp16 units, loss scale 65536, three iterations, an inf planted in unit 1 on iteration 2.
     Every share's update unscales on load; the policy for an overflow found after earlier units have
     been stepped: unit 1 and every unit stepped after it (unit 0) are skipped on the device, units 3
@@ -256,7 +303,7 @@ def test_scaled_gradients_and_overflow_while_stepping_during_backward(cuda, orac
     scaler = DynamicLossScaler(init_scale=65536.0, delayed_shift=1, scale_window=1000)
     flat, group, opt, coord, state = _fp16_units(
         cuda, num_units, unit_numel, offload, micro_batch_per_rank=micro_batches, unit_windows=windows,
-        gradacc_dtype=gradacc, loss_scaler=scaler)
+        gradacc_dtype=gradacc, loss_scaler=scaler, **_resident_kwargs(mode, micro_batches))
     expected_half = [half_bits(f).copy() for f in flat]
     gen = torch.Generator(device=cuda).manual_seed(9)
     seen_scales, overflows = [], []
@@ -300,8 +347,9 @@ def test_scaled_gradients_and_overflow_while_stepping_during_backward(cuda, orac
     assert overflows == [False, True, False]
 
 
-@pytest.mark.parametrize("offload,windows,gradacc", [(False, False, None), (True, True, None), (True, False, torch.float32)])
-def test_deferred_schedule_gives_a_global_decision(cuda, oracle, offload, windows, gradacc):
+@pytest.mark.parametrize("offload,windows,gradacc,mode", _with_resident_modes([
+    (False, False, None), (True, True, None), (True, False, torch.float32), (False, False, torch.float32)]))
+def test_deferred_schedule_gives_a_global_decision(cuda, oracle, offload, windows, gradacc, mode):
     """defer_to_forward: backward only accumulates and gathers statistics; one decision per
     iteration after the first unit's backward; the updates run during the next forward pass.
     Iteration 2 carries a nan in the LAST unit to run backward (unit 0): every unit, also those whose
@@ -313,7 +361,8 @@ def test_deferred_schedule_gives_a_global_decision(cuda, oracle, offload, window
     scaler = DynamicLossScaler(init_scale=4096.0, delayed_shift=1, scale_window=1000)
     flat, group, opt, coord, state = _fp16_units(
         cuda, num_units, unit_numel, offload, micro_batch_per_rank=micro_batches, unit_windows=windows,
-        gradacc_dtype=gradacc, loss_scaler=scaler, max_grad_norm=max_norm, defer_to_forward=True)
+        gradacc_dtype=gradacc, loss_scaler=scaler, max_grad_norm=max_norm, defer_to_forward=True,
+        **_resident_kwargs(mode, micro_batches))
     expected_half = [half_bits(f).copy() for f in flat]
     gen = torch.Generator(device=cuda).manual_seed(10)
 
