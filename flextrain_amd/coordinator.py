@@ -25,7 +25,10 @@ What changes because the optimizer runs on the GPU:
     unit's parameter buffer in HBM: no H2D copy of new parameters afterwards. A unit whose
     parameters are kept partly or wholly in pinned host memory (the reference's GPU part + CPU
     part, ``coordinator/parameter.py:470-519``) gets each element's new value in the piece that
-    holds it, written over the link by the same step.
+    holds it, written over the link by the same step;
+  * a unit whose master state is resident in HBM is stepped by one launch rather than a share per
+    micro-batch (``resident_shares``): the shares exist to spread host work or transfers, and it
+    has neither.
 Left out (other subsystems): the forward/backward alpha split with borrowed buffers, the NVMe
 tier, gradient reduce-scatter across ranks.
 
@@ -538,7 +541,7 @@ class FlexTrainOptsCoordinator:
 
     def _fwd_guard_parameters(self) -> None:
         """The forward pass that follows on the caller's stream reads the low-precision parameters the
-        offloaded step's kernels (on the engine's stream) have just written."""
+        step's kernels (on the offload engine's stream, or on the step stream) have just written."""
         if self._offload and not self._deferred_skip:
             self._optimizer.cpu_optimizer.stream_wait()
         self._caller_follows_steps()
