@@ -14,6 +14,7 @@
 #include <cmath>
 #include <map>
 #include <mutex>
+#include <type_traits>
 #include <unordered_map>
 
 #include "ft_internal.hpp"
@@ -243,7 +244,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         d.body_tiles = static_cast<uint32_t>(ntiles);
         d.hyper = hyper;
         d.c = c;
-        return launch_adam_multi(ma, GT, h != nullptr, HT, static_cast<unsigned>(ntiles) + 1u, stream);
+        return launch_adam_multi(ma, GT, h != nullptr, HT, hyper != nullptr, static_cast<unsigned>(ntiles) + 1u, stream);
     }
 
     if (ntiles > 0) {
@@ -264,12 +265,19 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         const size_t max_grid = 0x7fffffffu;  // one workgroup per tile; a larger count is split
         for (size_t tile0 = 0; tile0 < ntiles; tile0 += max_grid) {
             const size_t blocks = (ntiles - tile0 < max_grid) ? (ntiles - tile0) : max_grid;
-            if (ctl)
-                hipLaunchKernelGGL((ftk::adam_tile_kernel<GT, HT, true>), dim3(static_cast<unsigned>(blocks)),
-                                   dim3(ftk::kWave), lds, stream, a, static_cast<uint64_t>(tile0));
+            auto launch = [&](auto has_ctl, auto has_hyper) {
+                hipLaunchKernelGGL((ftk::adam_tile_kernel<GT, HT, decltype(has_ctl)::value, decltype(has_hyper)::value>),
+                                   dim3(static_cast<unsigned>(blocks)), dim3(ftk::kWave), lds, stream, a,
+                                   static_cast<uint64_t>(tile0));
+            };
+            if (ctl && hyper)
+                launch(std::true_type{}, std::true_type{});
+            else if (ctl)
+                launch(std::true_type{}, std::false_type{});
+            else if (hyper)
+                launch(std::false_type{}, std::true_type{});
             else
-                hipLaunchKernelGGL((ftk::adam_tile_kernel<GT, HT, false>), dim3(static_cast<unsigned>(blocks)),
-                                   dim3(ftk::kWave), lds, stream, a, static_cast<uint64_t>(tile0));
+                launch(std::false_type{}, std::false_type{});
             FT_HIP(hipGetLastError());
         }
     }
@@ -316,34 +324,44 @@ int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, 
 namespace {
 
 template <int GT, int HT>
-void launch_multi_typed(const ftk::AdamMultiArgs& a, unsigned workgroups, unsigned lds, hipStream_t stream)
+void launch_multi_typed(const ftk::AdamMultiArgs& a, bool with_hyper, unsigned workgroups, unsigned lds, hipStream_t stream)
 {
-    if (a.ctl)
-        hipLaunchKernelGGL((ftk::adam_multi_kernel<GT, HT, true>), dim3(workgroups), dim3(ftk::kWave), lds, stream, a);
+    auto launch = [&](auto has_ctl, auto has_hyper) {
+        hipLaunchKernelGGL((ftk::adam_multi_kernel<GT, HT, decltype(has_ctl)::value, decltype(has_hyper)::value>),
+                           dim3(workgroups), dim3(ftk::kWave), lds, stream, a);
+    };
+    if (a.ctl && with_hyper)
+        launch(std::true_type{}, std::true_type{});
+    else if (a.ctl)
+        launch(std::true_type{}, std::false_type{});
+    else if (with_hyper)
+        launch(std::false_type{}, std::true_type{});
     else
-        hipLaunchKernelGGL((ftk::adam_multi_kernel<GT, HT, false>), dim3(workgroups), dim3(ftk::kWave), lds, stream, a);
+        launch(std::false_type{}, std::false_type{});
 }
 
 template <int GT>
-void launch_multi_g(const ftk::AdamMultiArgs& a, bool with_half, int half_dtype, unsigned workgroups, hipStream_t stream)
+void launch_multi_g(const ftk::AdamMultiArgs& a, bool with_half, int half_dtype, bool with_hyper, unsigned workgroups,
+                    hipStream_t stream)
 {
     const unsigned lds = throttle_lds_bytes(48 + 4 * (GT == FT_F32 ? 4u : 2u));
-    if (!with_half) return launch_multi_typed<GT, -1>(a, workgroups, lds, stream);
-    if (half_dtype == FT_F16) return launch_multi_typed<GT, FT_F16>(a, workgroups, lds, stream);
-    return launch_multi_typed<GT, FT_BF16>(a, workgroups, lds, stream);
+    if (!with_half) return launch_multi_typed<GT, -1>(a, with_hyper, workgroups, lds, stream);
+    if (half_dtype == FT_F16) return launch_multi_typed<GT, FT_F16>(a, with_hyper, workgroups, lds, stream);
+    return launch_multi_typed<GT, FT_BF16>(a, with_hyper, workgroups, lds, stream);
 }
 
 }  // namespace
 
-// One launch over the segments collected in `a` (count of them, total workgroups).
-int launch_adam_multi(const ftk::AdamMultiArgs& a, int g_dtype, bool with_half, int half_dtype, unsigned workgroups,
-                      hipStream_t stream)
+// One launch over the segments collected in `a` (count of them, total workgroups). with_hyper: every
+// segment's scalars are read from its device record (all of them or none: two kernel variants).
+int launch_adam_multi(const ftk::AdamMultiArgs& a, int g_dtype, bool with_half, int half_dtype, bool with_hyper,
+                      unsigned workgroups, hipStream_t stream)
 {
     if (workgroups == 0) return FT_OK;
     switch (g_dtype) {
-        case FT_F32: launch_multi_g<FT_F32>(a, with_half, half_dtype, workgroups, stream); break;
-        case FT_F16: launch_multi_g<FT_F16>(a, with_half, half_dtype, workgroups, stream); break;
-        default: launch_multi_g<FT_BF16>(a, with_half, half_dtype, workgroups, stream); break;
+        case FT_F32: launch_multi_g<FT_F32>(a, with_half, half_dtype, with_hyper, workgroups, stream); break;
+        case FT_F16: launch_multi_g<FT_F16>(a, with_half, half_dtype, with_hyper, workgroups, stream); break;
+        default: launch_multi_g<FT_BF16>(a, with_half, half_dtype, with_hyper, workgroups, stream); break;
     }
     FT_HIP(hipGetLastError());
     return FT_OK;
@@ -617,19 +635,20 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
             return fth::fail(FT_EALIGN, "segment %d: a pointer is not aligned to its element size", i);
         if (sg.hyper && !aligned(sg.hyper, 16)) return fth::fail(FT_EALIGN, "segment %d: ft_adam_hyper_t must be 16-byte aligned", i);
     }
-    // Two batches fill side by side (with and without a low-precision copy: two kernel variants);
-    // a batch is launched when it holds kMultiMaxSegments segments or its grid is full.
+    // Four batches fill side by side (with and without a low-precision copy, scalars by value or from
+    // a device record: four kernel variants); a batch is launched when it holds kMultiMaxSegments
+    // segments or its grid is full.
     struct Batch {
         ftk::AdamMultiArgs a;
         int count = 0;
         unsigned workgroups = 0;
-    } batch[2];
+    } batch[4];
     auto flush = [&](int which) -> int {
         Batch& b = batch[which];
         if (b.count == 0) return FT_OK;
         for (int k = b.count; k < ftk::kMultiMaxSegments; ++k) b.a.first_wg[k] = 0xffffffffu;
         b.a.ctl = ctl;
-        const int r = fth::launch_adam_multi(b.a, g_dtype, which == 1, half_dtype, b.workgroups, stream);
+        const int r = fth::launch_adam_multi(b.a, g_dtype, (which & 1) != 0, half_dtype, (which & 2) != 0, b.workgroups, stream);
         b.count = 0;
         b.workgroups = 0;
         return r;
@@ -658,7 +677,7 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
             if (rc != FT_OK) return rc;
             continue;
         }
-        const int which = sg.half_out ? 1 : 0;
+        const int which = (sg.half_out ? 1 : 0) | (sg.hyper ? 2 : 0);
         const unsigned wgs = static_cast<unsigned>(body_tiles) + (edge ? 1u : 0u);
         if (batch[which].count == ftk::kMultiMaxSegments || batch[which].workgroups + static_cast<size_t>(wgs) > ftk::kMultiMaxWorkgroups)
             if ((rc = flush(which)) != FT_OK) return rc;
@@ -678,8 +697,9 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
         b.workgroups += wgs;
         ++b.count;
     }
-    if ((rc = flush(0)) != FT_OK) return rc;
-    return flush(1);
+    for (int which = 0; which < 4; ++which)
+        if ((rc = flush(which)) != FT_OK) return rc;
+    return FT_OK;
 }
 
 size_t ft_grad_stats_workspace_bytes(void) { return sizeof(ftk::StatsPartial) * kMaxStatsBlocks; }

@@ -45,8 +45,8 @@ int launch_adam(const ftk::AdamConsts& c, float* p, const void* g, int g_dtype, 
 size_t segment_head(const void* p, size_t n);
 
 // One launch of the many-segment update kernel over the table in `a` (see ft_types.hpp).
-int launch_adam_multi(const ftk::AdamMultiArgs& a, int g_dtype, bool with_half, int half_dtype, unsigned workgroups,
-                      hipStream_t stream);
+int launch_adam_multi(const ftk::AdamMultiArgs& a, int g_dtype, bool with_half, int half_dtype, bool with_hyper,
+                      unsigned workgroups, hipStream_t stream);
 
 int cu_count();  // compute units of the current device (cached)
 

@@ -174,16 +174,20 @@ __device__ __forceinline__ f32x4 load_g4(const void* g, uint64_t unit)
 // difference to a normal step, 0.835 against 0.833 ms; a skipped step costs 0.17 ms of workgroup
 // dispatch the first way and 0.40 ms the second). The low-precision copy is never written on a
 // skip: it has no input to copy from, so a caller that skips must not stage it.
-template <int GT, int HT, bool HAS_CTL>
+// HAS_HYPER: the step's scalars come from a.hyper (device memory, wave-uniform scalar loads) instead
+// of by value. A variant of its own rather than a test of the pointer: a branch in front of the
+// loads of the decision record and of the tile costs the common by-value path a dependent round of
+// scalar loads (and anything that looks like a memory write before them, even an empty asm
+// statement, turns the decision's scalar loads into vector loads: 0.81 -> 0.91 ms on the
+// mixed-precision step).
+template <int GT, int HT, bool HAS_CTL, bool HAS_HYPER>
 __global__ __launch_bounds__(kWave) void adam_tile_kernel(AdamArgs a, uint64_t tile0)
 {
-    AdamConsts c = a.c;
-    // The by-value scalars are pinned in scalar registers here, so that their loads go out with the
-    // other kernel arguments and are not sunk behind the test of a.hyper (a second, dependent
-    // round of scalar loads in front of every tile's vector loads).
-    asm volatile("" : "+s"(c.beta1), "+s"(c.beta2), "+s"(c.omb1), "+s"(c.omb2), "+s"(c.bias2), "+s"(c.eps), "+s"(c.step_size),
-                 "+s"(c.wd_coef), "+s"(c.grad_mult), "+s"(c.wd_mode));
-    if (a.hyper) c = *a.hyper;  // the step's scalars kept in device memory (wave-uniform loads)
+    AdamConsts c;
+    if constexpr (HAS_HYPER)
+        c = *a.hyper;
+    else
+        c = a.c;
     const uint64_t t0 = (tile0 + blockIdx.x) * kWave;  // first unit of the tile: wave-uniform
     const uint64_t i = t0 + threadIdx.x;
     if constexpr (HAS_CTL) {  // wave-uniform scalar loads: one decision per step
@@ -269,7 +273,7 @@ __global__ __launch_bounds__(256) void adam_scalar_kernel(AdamArgs a)
 // lane and round, through the same adam_element. In place only.
 typedef const char __attribute__((address_space(4))) * KernargBytes;
 
-template <int GT, int HT, bool HAS_CTL>
+template <int GT, int HT, bool HAS_CTL, bool HAS_HYPER>
 __global__ __launch_bounds__(kWave) void adam_multi_kernel(AdamMultiArgs a)
 {
     // Table entry k = (first workgroup of segment k) << 4 | k, ascending, unused entries all ones:
@@ -290,17 +294,20 @@ __global__ __launch_bounds__(kWave) void adam_multi_kernel(AdamMultiArgs a)
     typedef const AdamSegment __attribute__((address_space(4))) * SegPtr;
     const SegPtr sg = reinterpret_cast<SegPtr>(ka + __builtin_offsetof(AdamMultiArgs, seg) + s * sizeof(AdamSegment));
     AdamConsts c;
-    c.beta1 = sg->c.beta1;
-    c.beta2 = sg->c.beta2;
-    c.omb1 = sg->c.omb1;
-    c.omb2 = sg->c.omb2;
-    c.bias2 = sg->c.bias2;
-    c.eps = sg->c.eps;
-    c.step_size = sg->c.step_size;
-    c.wd_coef = sg->c.wd_coef;
-    c.grad_mult = sg->c.grad_mult;
-    c.wd_mode = sg->c.wd_mode;
-    if (const AdamConsts* hyper = sg->hyper) c = *hyper;  // the segment's scalars kept in device memory
+    if constexpr (HAS_HYPER) {  // every segment of the launch keeps its scalars in device memory
+        c = *sg->hyper;
+    } else {
+        c.beta1 = sg->c.beta1;
+        c.beta2 = sg->c.beta2;
+        c.omb1 = sg->c.omb1;
+        c.omb2 = sg->c.omb2;
+        c.bias2 = sg->c.bias2;
+        c.eps = sg->c.eps;
+        c.step_size = sg->c.step_size;
+        c.wd_coef = sg->c.wd_coef;
+        c.grad_mult = sg->c.grad_mult;
+        c.wd_mode = sg->c.wd_mode;
+    }
     if constexpr (HAS_CTL) {
         if (a.ctl->skip) return;
         c.grad_mult = a.ctl->grad_mult;

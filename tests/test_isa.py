@@ -1,0 +1,71 @@
+"""What the compiler made of the update kernel, checked on the gfx950 assembly (no GPU needed).
+
+The kernel's speed hangs on a few properties of the generated code that a source change can lose
+without any test of results noticing: the decision record and the by-value scalars must be read with
+scalar loads (a vector load of the record in front of the tile's loads, waited for before the
+branch, cost 13 % on the mixed-precision step once), the tile's loads must be non-temporal and its
+stores streaming buffer stores, and the straight-line tile code must not spill."""
+import os
+import re
+import subprocess
+
+import pytest
+
+from flextrain_amd import build
+
+pytestmark = pytest.mark.timeout(300)
+
+
+@pytest.fixture(scope="module")
+def kernels(tmp_path_factory):
+    """name -> assembly text of every kernel in ft_adam.hip, compiled with the library's flags."""
+    out = tmp_path_factory.mktemp("isa") / "ft_adam.s"
+    flags = [f for f in build.HIPCC_FLAGS if f != "-fPIC"]
+    cmd = [build.hipcc(), *flags, "-I", build.INCLUDE, "-I", build.CSRC, "--cuda-device-only", "-S",
+           os.path.join(build.CSRC, "ft_adam.hip"), "-o", str(out)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    text = out.read_text()
+    found = {}
+    for match in re.finditer(r"^(_ZN3ftk\w+):.*?\n(.*?)^\s*s_endpgm", text, re.S | re.M):
+        found[match.group(1)] = match.group(2)
+    assert found
+    return found
+
+
+def _tile_variants(kernels):
+    pattern = re.compile(r"adam_tile_kernelILi(\w+)ELi(\w+)ELb([01])ELb([01])E")
+    for name, body in kernels.items():
+        m = pattern.search(name)
+        if m:
+            yield name, m.group(1), m.group(2), m.group(3) == "1", m.group(4) == "1", body
+
+
+def test_every_tile_kernel_variant_is_there(kernels):
+    variants = {(g, h, c, y) for _, g, h, c, y, _ in _tile_variants(kernels)}
+    assert len(variants) == 3 * 3 * 2 * 2  # gradient type x copy type (none, fp16, bf16) x decision record x device scalars
+
+
+def test_uniform_values_come_through_scalar_loads(kernels):
+    """By-value variants: nothing wave-uniform is fetched with a vector load (those show up as
+    global loads with a scalar base register), and the decision record is read with s_load."""
+    for name, _, _, has_ctl, has_hyper, body in _tile_variants(kernels):
+        if has_hyper:
+            continue
+        uniform_vector_loads = re.findall(r"global_load_\w+\s+v[\[\d:\]]+, v\d+, s\[", body)
+        assert not uniform_vector_loads, (name, uniform_vector_loads)
+        scalar_record_loads = re.findall(r"s_load_dword\s+s\d+, s\[\d+:\d+\], 0x[04]\b", body)
+        assert (len(scalar_record_loads) >= 2) == has_ctl, (name, scalar_record_loads)
+
+
+def test_tile_traffic_is_streaming(kernels):
+    """Per-lane loads are all non-temporal, stores all streaming buffer stores; their number is that of
+    the arrays (plus the three copy-through pairs of a skipped out-of-place step)."""
+    for name, g, h, has_ctl, _, body in _tile_variants(kernels):
+        lane_loads = re.findall(r"global_load_dwordx[24]\s+v\[\d+:\d+\], v\[\d+:\d+\], off(.*)", body)
+        assert len(lane_loads) == 4 + (3 if has_ctl else 0) and all(" nt" in tail for tail in lane_loads), (name, lane_loads)
+        stores = re.findall(r"buffer_store_dwordx([24]) (.*)", body)
+        assert all(tail.rstrip().endswith("offen nt sc1") for _, tail in stores), (name, stores)
+        widths = [w for w, _ in stores]
+        assert widths.count("4") == 3 + (3 if has_ctl else 0) and widths.count("2") == (0 if h == "n1" else 1), (name, widths)
+        assert "global_store" not in body and "scratch_" not in body, name
