@@ -838,6 +838,12 @@ int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t 
         if (head > n) head = n;
         if (!aligned(static_cast<char*>(g) + head * gsz, gsz * 4))
             return fth::fail(FT_EALIGN, "acc and g must start at the same element offset modulo 4 of their buffers");
+        // A long buffer: on to the first tile boundary of acc (256 elements = 1 KiB of fp32), so that
+        // every tile's streaming stores cover whole cache lines (a multiple of 4 more: g stays aligned).
+        if (n - head >= 16 * 256) {
+            const size_t tile_bytes = 256 * asz;
+            head = ((tile_bytes - (reinterpret_cast<uintptr_t>(acc) & (tile_bytes - 1))) & (tile_bytes - 1)) / asz;
+        }
         nvec = (n - head) / 4;
     }
     ftk::StatsPartial* parts = nullptr;

@@ -756,9 +756,10 @@ __global__ __launch_bounds__(256) void reduce_wave_partials_kernel(const WavePar
     }
 }
 
-// Last launch of an accumulation pass (one block of 256): thread 0 takes the elements outside the
-// vector body one by one; with STATS the block then adds the second-level partials in a fixed tree
-// order, thread 0 adds the edge elements' share and writes or accumulates the result.
+// Last launch of an accumulation pass (one block of 256): the elements outside the vector body (up
+// to 255 in front of it, up to 3 behind) go one per thread and round; with STATS the block then adds
+// the second-level partials and every thread's edge share in a fixed tree order and thread 0 writes
+// or accumulates the result.
 template <int AT, int GT, bool ZERO, bool STATS>
 __global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, void* g, uint64_t head,
                                                                      uint64_t tail_begin, uint64_t n, float scale,
@@ -769,9 +770,9 @@ __global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, 
 {
     double s = 0.0;
     uint64_t b = 0;
-    for (uint64_t i = 0; threadIdx.x == 0 && i < n; ++i) {
-        if (i == head) i = tail_begin;
-        if (i >= n) break;
+    const uint64_t edge = head + (n - tail_begin);
+    for (uint64_t e = threadIdx.x; e < edge; e += 256) {
+        const uint64_t i = e < head ? e : tail_begin + (e - head);
         float gi;
         if constexpr (GT == FT_F32)
             gi = reinterpret_cast<const float*>(g)[i];
@@ -812,8 +813,8 @@ __global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, 
     if constexpr (STATS) {
         __shared__ double s_sum[256];
         __shared__ uint64_t s_bad[256];
-        double ps = 0.0;
-        uint64_t pb = 0;
+        double ps = s;   // this thread's edge elements, then its share of the partials
+        uint64_t pb = b;
         for (int i = threadIdx.x; i < nparts; i += 256) {
             ps += partials[i].sumsq;
             pb += partials[i].nonfinite;
@@ -828,11 +829,7 @@ __global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, 
             }
             __syncthreads();
         }
-        if (threadIdx.x == 0) {
-            s += s_sum[0];
-            b += s_bad[0];
-            publish_stats(s, b, out, accumulate, inv_scale, max_norm, ctl);
-        }
+        if (threadIdx.x == 0) publish_stats(s_sum[0], s_bad[0], out, accumulate, inv_scale, max_norm, ctl);
     }
 }
 

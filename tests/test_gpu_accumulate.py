@@ -25,7 +25,7 @@ def test_accumulate_matrix(cuda, oracle, acc_dtype, g_dtype, scale, zero):
     from flextrain_amd.loss_scaler import GradientGuard
     guard = GradientGuard(cuda)
     gen = torch.Generator(device=cuda).manual_seed(3)
-    for n, offset in ((1, 0), (5, 3), (1000, 1), (4096, 0), (300_007, 2)):
+    for n, offset in ((1, 0), (5, 3), (1000, 1), (4096, 0), (4099, 1), (70_001, 37), (300_007, 2)):
         A = torch.randn(n + offset + 8, device=cuda, generator=gen).to(acc_dtype)
         G = (torch.randn(n + offset + 8, device=cuda, generator=gen) * 0.1).to(g_dtype)
         a, g = A[offset:offset + n], G[offset:offset + n]
