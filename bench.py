@@ -373,6 +373,7 @@ def bench_pipeline(args, torch, dev) -> int:
 
     lib = _C.lib()
     n, mb = N_7B_LAYER, args.micro_batches
+    _C.check("ft_offload_set_window_piece", lib.ft_offload_set_window_piece(args.window_piece_mi << 20))
     if args.resident:
         return bench_pipeline_resident(args, torch, dev, Unit)
     units = min(args.layers, 24 + args.resident_units)  # 24 streamed layers = 58 GB of pinned state, inside what the box pins
@@ -432,7 +433,8 @@ def bench_pipeline(args, torch, dev) -> int:
         "config": {"workload": f"pipeline: coordinator schedule over {units} Llama-7B layers, {mb} shares per unit, "
                                "fp32 state in pinned host DRAM, bf16 grads and parameters on GPU",
                    "elements": total, "units": units, "micro_batches": mb, "chunk_elems": args.chunk_elems,
-                   "slots": args.slots, "unit_windows": args.windows, "resident_units": min(args.resident_units, units),
+                   "slots": args.slots, "unit_windows": args.windows, "window_piece_mi": args.window_piece_mi,
+                   "resident_units": min(args.resident_units, units),
                    "streamed_elements": streamed},
         "iteration_ms": [w * 1e3 for w in walls],
         "link": dict(link, achieved_each_way_gbps=one_way, achieved_total_gbps=2 * one_way,
@@ -699,6 +701,8 @@ def main() -> int:
     ap.add_argument("--layer-groups", action="store_true",
                     help="pipeline --resident: each layer as its nine tensors in two parameter groups (matrices with weight "
                          "decay, norms without), so that group boundaries cut shares into several step contexts")
+    ap.add_argument("--window-piece-mi", type=int, default=0,
+                    help="pipeline: elements (in Mi) per piece of a unit window's copies (0 = the library's default)")
     ap.add_argument("--resident-shares", type=int, default=0,
                     help="pipeline --resident: launches a resident unit's update is cut into (0 = the coordinator's default)")
     ap.add_argument("--step-stream", default="auto", choices=["auto", "on", "off"],

@@ -9,6 +9,7 @@
 #include <string.h>
 
 #include <chrono>
+#include <atomic>
 #include <deque>
 #include <mutex>
 #include <vector>
@@ -56,6 +57,7 @@ constexpr size_t kMaxPending = 8;
 // degradation of long bursts of copies that kMaxChunksPerStep guards against.
 constexpr size_t kWindowPieceElems = 256u * 1024u * 1024u;  // about 1 GiB per array and copy
 constexpr int kMaxWindows = 4;
+std::atomic<size_t> g_window_piece_elems{kWindowPieceElems};  // ft_offload_set_window_piece
 
 struct Window {
     float* dev[3] = {nullptr, nullptr, nullptr};
@@ -68,7 +70,11 @@ struct Window {
     size_t piece = 0;                // elements per copy: n cut into equal pieces, never a small tail
     uint64_t closed_at = 0;          // order of closing: the window closed longest ago is reused first
     std::vector<hipEvent_t> piece_done;
-    hipEvent_t k_done = nullptr, d2h_done = nullptr;
+    // Copy-back as pieces complete: elements of piece k stepped since it was last written back, and
+    // whether the host already holds what the device copy of piece k holds.
+    std::vector<size_t> piece_stepped;
+    std::vector<char> piece_clean;
+    hipEvent_t k_done = nullptr, d2h_done = nullptr, piece_stepped_ev = nullptr;
 };
 
 // Automatic choice of the transfer mode. Measured on MI355X / PCIe Gen5 x16: SDMA copies through
@@ -159,6 +165,7 @@ void destroy_engine(Engine* e)
         for (hipEvent_t ev : w.piece_done) (void)hipEventDestroy(ev);
         if (w.k_done) (void)hipEventDestroy(w.k_done);
         if (w.d2h_done) (void)hipEventDestroy(w.d2h_done);
+        if (w.piece_stepped_ev) (void)hipEventDestroy(w.piece_stepped_ev);
     }
     e->magic = 0;
     delete e;
@@ -526,11 +533,38 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
                               window->dev[2] + window_off, half_out, half_dtype, n,
                               static_cast<const ft_step_control_t*>(ctl), e->s_k, out[0], out[1], out[2]);
         if (rc != FT_OK) return rc;
-        // Only the kernel stream is touched: the copy streams carry the windows' large copies and
-        // nothing else (hundreds of small steps per iteration would otherwise add as many markers
-        // to the D2H stream).
+        // Only the kernel stream is touched by most steps: the copy streams carry the windows' large
+        // copies and nothing else (hundreds of small steps per iteration would otherwise add as many
+        // markers to the D2H stream). The step that completes a piece -- every element of it
+        // stepped since the piece was last written back -- sends that piece on its way back, so
+        // that the write-back of a window runs one piece, not one window, behind its steps.
         FT_HIP(hipEventRecord(e->ev_kernels, e->s_k));
         e->stepped = true;
+        if (!window->write_through) {
+            Window& w = *window;
+            const size_t first_piece = window_off / w.piece;
+            bool waited = false;
+            for (size_t k = first_piece; k <= last_piece; ++k) {
+                const size_t lo = k * w.piece, hi = (lo + w.piece < w.n) ? lo + w.piece : w.n;
+                const size_t a = window_off > lo ? window_off : lo, b = (window_off + n < hi) ? window_off + n : hi;
+                if (w.piece_clean[k]) {  // stepped again after its write-back: that copy is stale
+                    w.piece_clean[k] = 0;
+                    w.piece_stepped[k] = 0;
+                }
+                w.piece_stepped[k] += b - a;
+                if (w.piece_stepped[k] < hi - lo) continue;
+                if (!waited) {
+                    FT_HIP(hipEventRecord(w.piece_stepped_ev, e->s_k));
+                    FT_HIP(hipStreamWaitEvent(e->s_d2h, w.piece_stepped_ev, 0));
+                    waited = true;
+                }
+                for (int arr = 0; arr < 3; ++arr)
+                    FT_HIP(hipMemcpyAsync(reinterpret_cast<float*>(w.host[arr]) + lo, w.dev[arr] + lo, (hi - lo) * 4,
+                                          hipMemcpyDeviceToHost, e->s_d2h));
+                w.piece_clean[k] = 1;
+                w.piece_stepped[k] = 0;
+            }
+        }
         return FT_OK;
     }
     FT_HIP(hipEventRecord(e->ev_begin, in_staged ? e->s_h2d : e->s_k));
@@ -676,6 +710,7 @@ int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_
     Window& w = e->windows[pick];
     if (!w.k_done) FT_HIP(hipEventCreateWithFlags(&w.k_done, hipEventDisableTiming));
     if (!w.d2h_done) FT_HIP(hipEventCreateWithFlags(&w.d2h_done, hipEventDisableTiming));
+    if (!w.piece_stepped_ev) FT_HIP(hipEventCreateWithFlags(&w.piece_stepped_ev, hipEventDisableTiming));
     if (w.cap < n) {
         if (w.used) FT_HIP(hipEventSynchronize(w.d2h_done));  // its last write-back still reads the old arrays
         for (float*& d : w.dev) {
@@ -694,7 +729,8 @@ int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_
     }
     // Equal pieces of about kWindowPieceElems: a short last copy would be one of the small copies
     // that make the copy engines share (see kStagedMinElems).
-    size_t pieces = (n + kWindowPieceElems / 2) / kWindowPieceElems;
+    const size_t piece_elems = g_window_piece_elems.load();
+    size_t pieces = (n + piece_elems / 2) / piece_elems;
     if (pieces == 0) pieces = 1;
     const size_t piece = ((n + pieces - 1) / pieces + 3) / 4 * 4;
     pieces = (n + piece - 1) / piece;
@@ -717,6 +753,8 @@ int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_
     for (int a = 0; a < 3; ++a) w.host[a] = reinterpret_cast<uintptr_t>(host[a]);
     w.n = n;
     w.piece = piece;
+    w.piece_stepped.assign(pieces, 0);
+    w.piece_clean.assign(pieces, 0);  // nothing stepped yet, but a close without steps still copies back (as before)
     w.write_through = write_through != 0;
     w.open = true;
     *out_window = pick;
@@ -739,6 +777,7 @@ int ft_offload_window_close(void* handle, int window)
     FT_HIP(hipStreamWaitEvent(e->s_d2h, w.piece_done[pieces - 1], 0));
     Pending mine;
     for (size_t k = 0; k < pieces && !w.write_through; ++k) {
+        if (w.piece_clean[k]) continue;  // written back when its last element was stepped
         const size_t off = k * w.piece;
         const size_t cnt = (w.n - off < w.piece) ? (w.n - off) : w.piece;
         for (int a = 0; a < 3; ++a)
@@ -757,6 +796,13 @@ int ft_offload_window_close(void* handle, int window)
     w.used = true;
     w.closed_at = ++e->window_closes;
     return remember_writeback(e, mine);
+}
+
+int ft_offload_set_window_piece(size_t elems)
+{
+    if (elems != 0 && elems < (1u << 20)) return fth::fail(FT_EINVAL, "window pieces of fewer than 1 Mi elements are refused");
+    g_window_piece_elems = elems ? elems : kWindowPieceElems;
+    return FT_OK;
 }
 
 int ft_offload_set_mode(void* handle, int mode)

@@ -261,7 +261,8 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
  * the device with large copies and returns at once; until ft_offload_window_close, every
  * ft_offload_step whose p/m/v lie inside those arrays (same element offset in all three) runs as
  * a kernel on the device copy. write_through == 0: the kernels work in place on the device copy,
- * the host arrays are stale until the close has written all three back with large copies.
+ * the host arrays are stale until the close (a piece of them may be written back earlier, when the
+ * steps have covered it; the close writes back whatever is left).
  * write_through != 0: the kernels write their results straight to the host arrays (no copy back;
  * each element may be stepped at most once per window). A step may not straddle a window's edge.
  * At most 4 windows are open at a time (FT_EBUSY beyond). The reference has no counterpart: its
@@ -269,6 +270,15 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
 int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_v, size_t n, int write_through,
                            int* out_window);
 int ft_offload_window_close(void* handle, int window);
+/* Windows cross the link in equal pieces of about `elems` elements per array (0 = the default,
+ * 256 Mi: about 1 GiB per copy). A window of copy-back kind sends a piece on its way back as soon as
+ * every element of it has been stepped, so its write-back runs one piece behind its steps; what is
+ * left goes at the close. Smaller pieces shorten that lag and make more, smaller copies -- which is
+ * not free: measured on a 24-unit schedule, four pieces per unit gained 3.5 % with 8 and 16 steps
+ * per unit and halved the throughput with 32, as eight pieces did with 16 (the runtime then carries
+ * both directions on one copy engine). Measure before changing it. Applies to windows opened
+ * afterwards, on every handle. */
+int ft_offload_set_window_piece(size_t elems);
 int ft_offload_stream_wait(void* handle, void* stream, int what);
 int ft_offload_wait(void* handle);
 int ft_offload_elapsed_ms(void* handle, float* out_ms);
