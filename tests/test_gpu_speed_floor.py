@@ -1,0 +1,81 @@
+"""Speed floors for the kernels that carry the traffic, on the Llama-7B decoder-layer partition.
+
+Not a benchmark (bench.py is): a guard against a change that leaves results intact and costs
+bandwidth. Each case takes the FASTEST of 20 launches (HIP events) and asks for at least 80 % of
+8 TB/s in algorithmic bytes; the kernels run at 84-88 % on every machine measured, and the slip this
+guard exists for (the decision record read with vector loads in front of the tile's loads) ran at
+79 %."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+N = 202_383_360  # 4*4096^2 + 3*4096*11008 + 2*4096
+PEAK = 8.0e12
+FLOOR = 0.80
+
+
+def _fastest_ms(fn, launches=20, warmup=3):
+    for _ in range(warmup):
+        fn()
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
+    for start, stop in pairs:
+        start.record()
+        fn()
+        stop.record()
+    torch.cuda.synchronize()
+    return min(start.elapsed_time(stop) for start, stop in pairs)
+
+
+def _arrays(cuda, g_dtype):
+    from flextrain_amd.memory import allocate_device_arrays
+    p, m, v, g, h = allocate_device_arrays([(N, torch.float32)] * 3 + [(N, g_dtype), (N, torch.bfloat16)], cuda)
+    p.normal_(0, 0.02)
+    m.normal_(0, 1e-4)
+    v.uniform_(0, 1e-6)
+    g.normal_(0, 1e-3)
+    return p, g, m, v, h
+
+
+def _check(summary_line, what, ms, bytes_per_element):
+    frac = N * bytes_per_element / (ms * 1e-3) / PEAK
+    summary_line(f"speed floor, {what}: fastest of 20 launches {ms:.4f} ms = {100 * frac:.1f} % of 8 TB/s")
+    assert frac >= FLOOR, f"{what}: {ms:.4f} ms = {100 * frac:.1f} % of peak, floor {100 * FLOOR:.0f} %"
+
+
+@pytest.mark.parametrize("variant", ["by_value", "control_record", "device_scalars", "control_record_and_device_scalars"])
+def test_update_kernel(cuda, summary_line, variant):
+    from flextrain_amd import FlexTrainCPUAdam
+    p, g, m, v, h = _arrays(cuda, torch.float16 if "control" in variant else torch.bfloat16)
+    eng = FlexTrainCPUAdam(lr=1e-4)
+    group = {"step": 100}
+    if "device_scalars" in variant:
+        eng.make_capturable(group, cuda)
+        group["hyper_record"].fill(group).sync()
+    control = torch.tensor([0.0, 1.0 / 65536, 0.0, 1.0], device=cuda) if "control" in variant else None
+    ms = _fastest_ms(lambda: eng._step(group, h, p, g, m, v, control=control))
+    _check(summary_line, f"update ({variant})", ms, 28)
+
+
+def test_update_of_sixteen_contexts_in_one_launch(cuda, summary_line):
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.param_group import StepContext
+    p, g, m, v, h = _arrays(cuda, torch.bfloat16)
+    eng = FlexTrainCPUAdam(lr=1e-4)
+    cuts = sorted(torch.randint(1, N - 1, (15,), generator=torch.Generator().manual_seed(3)).tolist())
+    groups = [{"step": 100, "weight_decay": 0.01}, {"step": 37, "weight_decay": 0.0}]
+    contexts = [StepContext(groups[k % 2], h[lo:hi], p[lo:hi], g[lo:hi], [m[lo:hi], v[lo:hi]])
+                for k, (lo, hi) in enumerate(zip([0] + cuts, cuts + [N]))]
+    ms = _fastest_ms(lambda: eng.step(contexts))
+    _check(summary_line, "update, 16 ragged contexts in one launch", ms, 28)
+
+
+def test_accumulate_and_clear(cuda, summary_line):
+    from flextrain_amd.loss_scaler import GradientGuard
+    from flextrain_amd.memory import allocate_device_arrays
+    acc, g = allocate_device_arrays([(N, torch.float32), (N, torch.bfloat16)], cuda)
+    acc.zero_()
+    g.zero_()
+    guard = GradientGuard(cuda)
+    ms = _fastest_ms(lambda: guard.accumulate(acc, g, zero_grads=True))
+    _check(summary_line, "accumulate + clear", ms, 12)
