@@ -27,7 +27,7 @@ def kernels(tmp_path_factory):
     assert res.returncode == 0, res.stderr
     text = out.read_text()
     found = {}
-    for match in re.finditer(r"^(_ZN3ftk\w+):.*?\n(.*?)^\s*s_endpgm", text, re.S | re.M):
+    for match in re.finditer(r"^(_ZN3ftk\w+):.*?\n(.*?)^\.Lfunc_end\d+:", text, re.S | re.M):
         found[match.group(1)] = match.group(2)
     assert found
     return found
@@ -69,3 +69,36 @@ def test_tile_traffic_is_streaming(kernels):
         widths = [w for w, _ in stores]
         assert widths.count("4") == 3 + (3 if has_ctl else 0) and widths.count("2") == (0 if h == "n1" else 1), (name, widths)
         assert "global_store" not in body and "scratch_" not in body, name
+
+
+def test_no_kernel_spills(kernels):
+    for name, body in kernels.items():
+        assert "scratch_" not in body, name
+
+
+def test_statistics_pass_has_a_streaming_and_a_caching_load_path(kernels):
+    """The statistics pass reads the part of the gradients that the update will want again with
+    caching buffer loads and everything else with non-temporal loads: both instructions must have
+    survived (a compiler that merges the two branches drops the streaming hint)."""
+    seen = 0
+    for name, body in kernels.items():
+        if "grad_stats_kernel" not in name:
+            continue
+        seen += 1
+        assert re.search(r"global_load_dwordx4 .* nt", body), name
+        assert re.search(r"buffer_load_dwordx4 ", body), name
+    assert seen == 3  # one per gradient type
+
+
+def test_many_segment_kernel_keeps_its_table_in_scalar_registers(kernels):
+    """The segment search is scalar compares and selects over the kernel arguments; the segment's
+    record comes through scalar loads at a computed offset (no private copy of the table, which
+    would show up as scratch or as vector loads of the arguments)."""
+    seen = 0
+    for name, body in kernels.items():
+        if "adam_multi_kernel" not in name:
+            continue
+        seen += 1
+        assert len(re.findall(r"s_cselect_b32", body)) >= 15, name
+        assert re.search(r"s_load_dwordx\d+ s\[\d+:\d+\], s\[\d+:\d+\], s\d+", body), name  # register offset: the computed record address
+    assert seen == 3 * 3 * 2 * 2
