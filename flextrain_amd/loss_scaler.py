@@ -30,6 +30,14 @@ CONSECUTIVE_HYSTERESIS = 'consecutive_hysteresis'
 MIN_LOSS_SCALE = 'min_scale'
 
 
+def to_python_float(tensor: torch.Tensor) -> float:
+    """One-element tensor to a Python number (reference ``loss_scaler.py:23-27``)."""
+    if hasattr(tensor, "item"):
+        return tensor.item()
+    assert tensor.nelement() == 1
+    return tensor[0]
+
+
 class LossScalerBase(ABC):
     """Holds the current scale (reference ``loss_scaler.py:30-49``)."""
 
@@ -58,6 +66,12 @@ class LossScaler(LossScalerBase):
         super().__init__(scale)
 
     def has_overflow(self, params):
+        return False
+
+    @staticmethod
+    def _has_inf_or_nan(x):
+        """A static scale never reports an overflow (reference ``:65-66``, there a method without
+        ``self``; callable both ways here)."""
         return False
 
 

@@ -3,7 +3,7 @@ import numpy as np
 import pytest
 import torch
 
-from flextrain_amd.loss_scaler import DynamicLossScaler, LossScaler, create_loss_scaler
+from flextrain_amd.loss_scaler import DynamicLossScaler, LossScaler, create_loss_scaler, to_python_float
 
 
 def run(scaler, overflows):
@@ -57,6 +57,9 @@ def test_static_scaler_and_factory():
     s = LossScaler(128.0)
     s.update_scale(True)
     assert s.loss_scale == 128.0 and not s.dynamic and s.has_overflow(None) is False
+    assert LossScaler._has_inf_or_nan(torch.tensor(float("inf"))) is False and s._has_inf_or_nan(None) is False
+    assert to_python_float(torch.tensor([2.5])) == 2.5
+    assert s.scale_gradient(None, (torch.ones(2),), None)[0].tolist() == [128.0, 128.0]
     d = create_loss_scaler(torch.float16)
     assert isinstance(d, DynamicLossScaler) and d.loss_scale == 65536 and d.delayed_shift == 2 and d.scale_window == 1000
     st = create_loss_scaler(torch.float16, dynamic_loss_scaling=False, initial_scale_power=8)
