@@ -336,8 +336,8 @@ struct LinkProbe {
     {
         *gbps = 0.0;
         for (int lanes = 1; lanes <= kLanes; ++lanes)
-            for (int round = 0; round < 2; ++round) {  // round 0 warms up
-                const int reps = round == 0 ? 1 : iters * (kLanes / lanes);
+            for (int timed = 0; timed < 2; ++timed) {  // the first pass warms up
+                const int reps = timed == 0 ? 1 : iters * (kLanes / lanes);
                 const auto t0 = std::chrono::steady_clock::now();
                 for (int i = 0; i < reps; ++i)
                     for (int l = 0; l < lanes; ++l)
