@@ -348,7 +348,7 @@ struct LinkProbe {
                 const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
                 const int dirs = (mask & 1) + ((mask >> 1) & 1);
                 const double rate = static_cast<double>(bytes) * lanes * reps * dirs / sec / 1e9;
-                if (round == 1 && rate > *gbps) *gbps = rate;
+                if (timed == 1 && rate > *gbps) *gbps = rate;
             }
         return FT_OK;
     }
