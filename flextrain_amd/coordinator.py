@@ -239,9 +239,11 @@ class FlexTrainOptsCoordinator:
         # Stepping during backward: two gradient buffers trade places every unit, [0] receives the
         # unit in backward, [1] holds the finished gradients of the unit being stepped. Deferred:
         # every unit keeps a buffer of its own until its update, one iteration later.
+        # (Separately aligned arrays, not rows of one matrix: a unit length that is no multiple of the
+        # vector width would leave every second row off its alignment.)
         self._gpu_bwd_grad_buffers = RotateContainer(tuple(
-            allocate_memory_chunks(self._unit_numel, 2, gradacc_dtype, device))) if not self._defer else None
-        self._unit_grads = allocate_memory_chunks(self._unit_numel, self._num_units, gradacc_dtype, device) \
+            allocate_device_arrays([(self._unit_numel, gradacc_dtype)] * 2, device))) if not self._defer else None
+        self._unit_grads = allocate_device_arrays([(self._unit_numel, gradacc_dtype)] * self._num_units, device) \
             if self._defer else None
         self._bwd_unit = -1  # deferred: the unit whose backward is running
         # When gradients are accumulated in a wider type than backward produces them in, backward
@@ -251,7 +253,7 @@ class FlexTrainOptsCoordinator:
         self._gpu_bwd_extra_grads = None
         if self._gradacc_dtype_incompatible:
             from .loss_scaler import GradientGuard
-            self._gpu_bwd_extra_grads = allocate_memory_chunks(self._unit_numel, 1, device_dtype, device)[0]
+            self._gpu_bwd_extra_grads = allocate_device_arrays([(self._unit_numel, device_dtype)], device)[0]
             self._guard = self._iter_guard if self._iter_guard is not None else GradientGuard(device)
 
         # [master | exp_avg | exp_avg_sq] per unit.
