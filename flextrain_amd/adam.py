@@ -247,8 +247,9 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             _C.current_stream_ptr()))
         if blocking is None or blocking:
             _C.check("ft_offload_wait", self._lib.ft_offload_wait(engine))
-        elif guard_stream and (gradient.is_cuda or (half_parameter is not None and half_parameter.is_cuda)):
-            # later work on the caller's stream may overwrite the gradients or read the new copy
+        elif guard_stream and (gradient.is_cuda or (half_parameter is not None and half_parameter.is_cuda) or control is not None):
+            # later work on the caller's stream may overwrite the gradients, read the new copy, or be
+            # given the control record's memory once the caller lets go of it
             _C.check("ft_offload_stream_wait", self._lib.ft_offload_stream_wait(engine, _C.current_stream_ptr(), 0))
 
     def _step_many(self, step_contexts, grad_mult: float = 1.0, control: Optional[Tensor] = None) -> None:
