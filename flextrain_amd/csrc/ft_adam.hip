@@ -835,8 +835,8 @@ int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t 
     if (n > 0) {
         if (!aligned(acc, asz) || !aligned(g, gsz)) return fth::fail(FT_EALIGN, "a pointer is not aligned to its element size");
         head = ((asz * 4 - (reinterpret_cast<uintptr_t>(acc) & (asz * 4 - 1))) & (asz * 4 - 1)) / asz;
-        if (head > n) head = n;
-        if (!aligned(static_cast<char*>(g) + head * gsz, gsz * 4))
+        if (head > n) head = n;  // shorter than the way to the first boundary: edge elements only
+        if (head < n && !aligned(static_cast<char*>(g) + head * gsz, gsz * 4))
             return fth::fail(FT_EALIGN, "acc and g must start at the same element offset modulo 4 of their buffers");
         // A long buffer: on to the first tile boundary of acc (256 elements = 1 KiB of fp32), so that
         // every tile's streaming stores cover whole cache lines (a multiple of 4 more: g stays aligned).
