@@ -3,6 +3,8 @@ offsets per array (equal offsets take the vector path with head and tail launche
 all-scalar path), every gradient / copy-out type, both decay modes, bias correction on and off,
 host-side multipliers, device-side control records, special values sprinkled in. Bit-exact bar
 (the documented tolerance is 2 ULP / 1 ULP; the kernels are written to hit 0)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -20,7 +22,7 @@ def _bits32(t):
     return to_np(t).view(np.uint32)
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("FT_FUZZ_SEEDS", "6"))))
 def test_random_cases_bit_exact(cuda, oracle, seed):
     from flextrain_amd import FlexTrainCPUAdam
     rng = np.random.default_rng(1000 + seed)
@@ -105,7 +107,7 @@ def test_random_cases_bit_exact(cuda, oracle, seed):
     assert worst_cases == 40
 
 
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("FT_FUZZ_SEEDS", "4"))))
 def test_random_many_context_calls_bit_exact(cuda, oracle, seed):
     """Seeded random calls of the many-contexts launch: 1 to 40 contexts of random length (a few
     elements to a few hundred thousand), random gaps between them in the flat buffers (so every
