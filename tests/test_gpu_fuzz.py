@@ -1,7 +1,8 @@
 """Seeded random cases of the resident update against the oracle: random lengths, random element
 offsets per array (equal offsets take the vector path with head and tail launches, unequal ones the
 all-scalar path), every gradient / copy-out type, both decay modes, bias correction on and off,
-host-side multipliers, device-side control records, special values sprinkled in. Bit-exact bar
+host-side multipliers, device-side control records, the step's scalars by value or in a device record,
+special values sprinkled in. Bit-exact bar
 (the documented tolerance is 2 ULP / 1 ULP; the kernels are written to hit 0)."""
 import os
 
@@ -78,14 +79,18 @@ def test_random_cases_bit_exact(cuda, oracle, seed):
                              half_dtype=CODE[h_dtype] if h_dtype is not None else F16)
 
         eng = FlexTrainCPUAdam(adamw_mode=adamw, **hp)
-        kw = {}
-        if mode == "mult":
+        kw, group = {}, {"step": step}
+        in_record = rng.random() < 0.35  # the step's scalars read from device memory instead of passed by value
+        if in_record:
+            eng.make_capturable(group, cuda)
+            group["hyper_record"].fill(group, grad_mult=grad_mult if mode == "mult" else 1.0).sync()
+        elif mode == "mult":
             kw["grad_mult"] = grad_mult
-        elif control is not None:
+        if control is not None:
             kw["control"] = control
-        eng._step({"step": step}, h, p, g, m, v, **kw)
+        eng._step(group, h, p, g, m, v, **kw)
 
-        tag = (seed, case, n, offs, str(g_dtype), str(h_dtype), adamw, hp, step, mode)
+        tag = (seed, case, n, offs, str(g_dtype), str(h_dtype), adamw, hp, step, mode, in_record)
         # NaN payloads: compare bits where finite, NaN-ness where not
         for name, got, want in (("p", p, pn), ("m", m, mn), ("v", v, vn)):
             gbits, wbits = _bits32(got), want.view(np.uint32)
