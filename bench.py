@@ -373,7 +373,6 @@ def bench_pipeline(args, torch, dev) -> int:
 
     lib = _C.lib()
     n, mb = N_7B_LAYER, args.micro_batches
-    _C.check("ft_offload_set_window_piece", lib.ft_offload_set_window_piece(args.window_piece_mi << 20))
     if args.resident:
         return bench_pipeline_resident(args, torch, dev, Unit)
     units = min(args.layers, 24 + args.resident_units)  # 24 streamed layers = 58 GB of pinned state, inside what the box pins
@@ -385,6 +384,7 @@ def bench_pipeline(args, torch, dev) -> int:
                             aligned_unit_numel=n, offload=True, **{k: HP[k] for k in ("lr", "betas", "eps", "weight_decay")})
         opt.cpu_optimizer._offload_chunk = args.chunk_elems
         opt.cpu_optimizer._offload_slots = args.slots
+        opt.cpu_optimizer._offload_window_piece = args.window_piece_mi << 20
         try:
             coord = FlexTrainOptsCoordinator()
             coord.initialize(opt, flat, mb, offload=True,

@@ -67,7 +67,7 @@ EXPORTS = {
     "ft_pinned_free": (c_int, [c_void_p]),
     "ft_offload_create": (c_int, [c_size_t, c_int, POINTER(c_void_p)]),
     "ft_offload_set_mode": (c_int, [c_void_p, c_int]),
-    "ft_offload_set_window_piece": (c_int, [c_size_t]),
+    "ft_offload_set_window_piece": (c_int, [c_void_p, c_size_t]),
     "ft_offload_destroy": (c_int, [c_void_p]),
     "ft_offload_step": (c_int, [c_void_p, c_int, c_uint64, c_float, c_float, c_float, c_float, c_float, c_int,
                                 c_float, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int,

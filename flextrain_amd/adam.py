@@ -103,6 +103,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
         offload_chunk_elems: int = DEFAULT_OFFLOAD_CHUNK,
         offload_slots: int = DEFAULT_OFFLOAD_SLOTS,
         offload_mode: int = 0,
+        offload_window_piece_elems: int = 0,
         should_log: bool = False,
         **kwargs,
     ):
@@ -121,6 +122,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
         self._offload_chunk = int(offload_chunk_elems)
         self._offload_slots = int(offload_slots)
         self._offload_mode = int(offload_mode)  # FT_OFFLOAD_* of include/ft_adam.h; 0 = automatic
+        self._offload_window_piece = int(offload_window_piece_elems)  # elements per piece of a window's copies; 0 = default
         self._engine: Optional[ctypes.c_void_p] = None
         _C.check("ft_adam_create", self._lib.ft_adam_create(
             self.opt_id, lr, betas[0], betas[1], eps, weight_decay, int(bool(adamw_mode)), int(bool(should_log))))
@@ -150,6 +152,7 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             _C.check("ft_offload_create", self._lib.ft_offload_create(
                 self._offload_chunk, self._offload_slots, ctypes.byref(handle)))
             _C.check("ft_offload_set_mode", self._lib.ft_offload_set_mode(handle, self._offload_mode))
+            _C.check("ft_offload_set_window_piece", self._lib.ft_offload_set_window_piece(handle, self._offload_window_piece))
             self._engine = handle
         return self._engine
 

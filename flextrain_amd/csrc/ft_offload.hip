@@ -9,7 +9,6 @@
 #include <string.h>
 
 #include <chrono>
-#include <atomic>
 #include <deque>
 #include <mutex>
 #include <vector>
@@ -57,7 +56,6 @@ constexpr size_t kMaxPending = 8;
 // degradation of long bursts of copies that kMaxChunksPerStep guards against.
 constexpr size_t kWindowPieceElems = 256u * 1024u * 1024u;  // about 1 GiB per array and copy
 constexpr int kMaxWindows = 4;
-std::atomic<size_t> g_window_piece_elems{kWindowPieceElems};  // ft_offload_set_window_piece
 
 struct Window {
     float* dev[3] = {nullptr, nullptr, nullptr};
@@ -115,6 +113,7 @@ struct Engine {
     std::vector<hipEvent_t> free_events;
     Window windows[kMaxWindows];
     uint64_t window_closes = 0;
+    size_t window_piece_elems = kWindowPieceElems;  // ft_offload_set_window_piece
 };
 
 Engine* as_engine(void* h)
@@ -729,7 +728,7 @@ int ft_offload_window_open(void* handle, void* host_p, void* host_m, void* host_
     }
     // Equal pieces of about kWindowPieceElems: a short last copy would be one of the small copies
     // that make the copy engines share (see kStagedMinElems).
-    const size_t piece_elems = g_window_piece_elems.load();
+    const size_t piece_elems = e->window_piece_elems;
     size_t pieces = (n + piece_elems / 2) / piece_elems;
     if (pieces == 0) pieces = 1;
     const size_t piece = ((n + pieces - 1) / pieces + 3) / 4 * 4;
@@ -798,10 +797,13 @@ int ft_offload_window_close(void* handle, int window)
     return remember_writeback(e, mine);
 }
 
-int ft_offload_set_window_piece(size_t elems)
+int ft_offload_set_window_piece(void* handle, size_t elems)
 {
+    Engine* e = as_engine(handle);
+    if (!e) return fth::fail(FT_ENOENT, "not an offload handle");
+    std::lock_guard<std::mutex> lock(e->mu);
     if (elems != 0 && elems < (1u << 20)) return fth::fail(FT_EINVAL, "window pieces of fewer than 1 Mi elements are refused");
-    g_window_piece_elems = elems ? elems : kWindowPieceElems;
+    e->window_piece_elems = elems ? elems : kWindowPieceElems;
     return FT_OK;
 }
 

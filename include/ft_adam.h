@@ -274,11 +274,11 @@ int ft_offload_window_close(void* handle, int window);
  * 256 Mi: about 1 GiB per copy). A window of copy-back kind sends a piece on its way back as soon as
  * every element of it has been stepped, so its write-back runs one piece behind its steps; what is
  * left goes at the close. Smaller pieces shorten that lag and make more, smaller copies -- which is
- * not free: measured on a 24-unit schedule, four pieces per unit gained 3.5 % with 8 and 16 steps
- * per unit and halved the throughput with 32, as eight pieces did with 16 (the runtime then carries
- * both directions on one copy engine). Measure before changing it. Applies to windows opened
- * afterwards, on every handle. */
-int ft_offload_set_window_piece(size_t elems);
+ * not free. Measured on a schedule of 24 units of 202 M elements: two pieces per unit gained 1.5-2.7 %
+ * with 4 to 32 steps per unit; four pieces gained 3.5 % with 8 and 16 steps per unit and halved the
+ * throughput with 32, as eight pieces did with 16 (the runtime then carries both directions on one
+ * copy engine). Measure before changing it. Applies to windows this handle opens afterwards. */
+int ft_offload_set_window_piece(void* handle, size_t elems);
 int ft_offload_stream_wait(void* handle, void* stream, int what);
 int ft_offload_wait(void* handle);
 int ft_offload_elapsed_ms(void* handle, float* out_ms);

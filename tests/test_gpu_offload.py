@@ -308,34 +308,29 @@ def test_window_pieces_go_back_as_their_steps_complete(cuda, oracle):
     stepped, the rest at the close; a piece stepped again after its write-back goes back again.
     Shares in scrambled order, one of them stepped a second time; the host arrays hold the oracle's
     result after the close, whichever way each piece travelled."""
-    from flextrain_amd import FlexTrainCPUAdam, _C
-    lib = _C.lib()
+    from flextrain_amd import FlexTrainCPUAdam
     share, shares = 1 << 19, 7
     n = share * shares  # 3.5 Mi elements: four pieces of 0.875 Mi, none aligned with the shares
-    _C.check("ft_offload_set_window_piece", lib.ft_offload_set_window_piece(1 << 20))
-    try:
-        with pytest.raises(ValueError, match="refused"):
-            _C.check("ft_offload_set_window_piece", lib.ft_offload_set_window_piece(4096))
-        eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 16, **HP)
-        p, m, v = _host_state(n, seed=77)
-        g = (torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16)
-        h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
-        pn, mn, vn, hn = _oracle(oracle, p, g, m, v, 4, torch.bfloat16)
-        again = slice(1 * share, 2 * share)  # share 1 once more, at step 5, after its pieces have gone back
-        ps, ms, vs, hs = pn[again].copy(), mn[again].copy(), vn[again].copy(), hn[again].copy()
-        oracle.adam_step(ps, to_np(g[again]), ms, vs, step=5, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
-                         weight_decay=HP["weight_decay"], g_dtype=CODE[torch.bfloat16], half_out=hs, half_dtype=CODE[torch.bfloat16])
-        pn[again], mn[again], vn[again], hn[again] = ps, ms, vs, hs
-        token = eng.open_window(p, m, v)
-        for k in (3, 0, 6, 1, 5, 2, 4):
-            sl = slice(k * share, (k + 1) * share)
-            eng._step({"step": 4}, h[sl], p[sl], g[sl], m[sl], v[sl], blocking=False)
-        eng._step({"step": 5}, h[again], p[again], g[again], m[again], v[again], blocking=False)
-        eng.close_window(token)
-        eng.synchronize()
-        _assert_equal_bits("window in pieces", p, m, v, h, (pn, mn, vn, hn), torch.bfloat16)
-    finally:
-        _C.check("ft_offload_set_window_piece", lib.ft_offload_set_window_piece(0))
+    with pytest.raises(ValueError, match="refused"):
+        FlexTrainCPUAdam(offload_window_piece_elems=4096, **HP)._offload_engine()
+    eng = FlexTrainCPUAdam(offload_chunk_elems=1 << 16, offload_window_piece_elems=1 << 20, **HP)
+    p, m, v = _host_state(n, seed=77)
+    g = (torch.randn(n, device=cuda) * 1e-3).to(torch.bfloat16)
+    h = torch.zeros(n, dtype=torch.bfloat16, device=cuda)
+    pn, mn, vn, hn = _oracle(oracle, p, g, m, v, 4, torch.bfloat16)
+    again = slice(1 * share, 2 * share)  # share 1 once more, at step 5, after its pieces have gone back
+    ps, ms, vs, hs = pn[again].copy(), mn[again].copy(), vn[again].copy(), hn[again].copy()
+    oracle.adam_step(ps, to_np(g[again]), ms, vs, step=5, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
+                     weight_decay=HP["weight_decay"], g_dtype=CODE[torch.bfloat16], half_out=hs, half_dtype=CODE[torch.bfloat16])
+    pn[again], mn[again], vn[again], hn[again] = ps, ms, vs, hs
+    token = eng.open_window(p, m, v)
+    for k in (3, 0, 6, 1, 5, 2, 4):
+        sl = slice(k * share, (k + 1) * share)
+        eng._step({"step": 4}, h[sl], p[sl], g[sl], m[sl], v[sl], blocking=False)
+    eng._step({"step": 5}, h[again], p[again], g[again], m[again], v[again], blocking=False)
+    eng.close_window(token)
+    eng.synchronize()
+    _assert_equal_bits("window in pieces", p, m, v, h, (pn, mn, vn, hn), torch.bfloat16)
 
 
 def test_write_through_window(cuda, oracle):

@@ -32,12 +32,13 @@ def test_random_offloaded_steps(cuda, oracle, seed):
     from flextrain_amd import FlexTrainCPUAdam
     from flextrain_amd.memory import pinned_empty
     rng = np.random.default_rng(10_000 + seed)
-    total = int(rng.integers(50_000, 1_200_000))
+    piece = int(rng.choice([0, 1 << 20]))  # windows in one piece, or in pieces of about 1 Mi elements
+    total = int(rng.integers(50_000, 3_200_000 if piece else 1_200_000))
     chunk = 1 << int(rng.integers(14, 19))
     slots, mode = int(rng.integers(2, 5)), int(rng.integers(0, 5))
     half_dtype = [torch.float16, torch.bfloat16][int(rng.integers(0, 2))]
-    print(f"[offload fuzz] seed={seed} total={total} chunk={chunk} slots={slots} mode={mode} half={half_dtype}", flush=True)
-    eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=slots, offload_mode=mode, **HP)
+    print(f"[offload fuzz] seed={seed} total={total} chunk={chunk} slots={slots} mode={mode} piece={piece} half={half_dtype}", flush=True)
+    eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_slots=slots, offload_mode=mode, offload_window_piece_elems=piece, **HP)
     P, M, V = (pinned_empty(total, torch.float32) for _ in range(3))
     P.copy_(torch.from_numpy(rng.normal(0, 0.02, total).astype(np.float32)))
     M.copy_(torch.from_numpy(rng.normal(0, 1e-4, total).astype(np.float32)))
