@@ -207,8 +207,8 @@ def test_wider_accumulation_type(cuda, oracle):
         assert max_ulp(to_np(v), vn) == 0 and max_ulp(half_bits(flat[u]), hn, bf16=True) == 0
 
 
-@pytest.mark.parametrize("offload", [True, False])
-def test_state_files_resume_bit_exact(cuda, tmp_path, offload):
+@pytest.mark.parametrize("offload,resident_units", [(True, 0), (False, 0), (True, 2)])
+def test_state_files_resume_bit_exact(cuda, tmp_path, offload, resident_units):
     """Save the units' [master | m | v] blocks as swap-format files after one iteration, wreck the
     live state, load, run a second iteration: same bits as a run that never stopped."""
     import os
@@ -226,7 +226,7 @@ def test_state_files_resume_bit_exact(cuda, tmp_path, offload):
         opt = FlexTrainAdam([group], lr=1e-3, unit_parameter_map={u: _Unit([params[u]]) for u in range(num_units)},
                             aligned_unit_numel=unit_numel, offload=offload)
         coord = FlexTrainOptsCoordinator()
-        coord.initialize(opt, flat, micro_batches, offload=offload)
+        coord.initialize(opt, flat, micro_batches, offload=offload, resident_units=resident_units)
         return flat, group, opt, coord
 
     def iterate(opt, coord, seed):
