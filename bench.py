@@ -82,6 +82,18 @@ def _host_description():
     return {"cpu_model": model, "logical_cpus": os.cpu_count(), "numa_nodes": len(glob.glob("/sys/devices/system/node/node[0-9]*")) or 1}
 
 
+def _device_description(torch, dev):
+    """What the runtime says about the GPU the figures were measured on (the roofline's peak is the
+    published 8 TB/s; the memory clock and bus width the driver reports are listed beside it)."""
+    props = torch.cuda.get_device_properties(dev)
+    out = {"name": props.name, "compute_units": props.multi_processor_count, "memory_gb": round(props.total_memory / 1e9, 1)}
+    for key in ("gcnArchName", "memory_clock_rate", "memory_bus_width", "L2_cache_size"):
+        value = getattr(props, key, None)
+        if value is not None:
+            out[key] = value
+    return out
+
+
 CPU_WARMUPS = 3
 
 
@@ -834,6 +846,7 @@ def main() -> int:
                    "copy_dtype": "bfloat16", "bytes_per_element": bytes_per_elem},
         "hbm_gbps": achieved,
         "hbm_frac_of_peak": achieved / HBM_PEAK_GBPS,
+        "device": _device_description(torch, dev),
         "roofline": {
             "bound": "hbm", "kernel": "adam_tile_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
