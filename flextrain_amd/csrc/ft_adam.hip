@@ -223,7 +223,39 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         return FT_OK;
     };
 
-    if (!vec_ok) return scalar_part(0, n);
+    if (!vec_ok) {
+        // Arrays whose alignments disagree: whole tiles behind p's own head still go through a tile
+        // kernel (one that assumes element alignment only), the rest element by element.
+        const size_t head4 = ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4;
+        const size_t rhead = head4 < n ? head4 : n;
+        const size_t rtiles = (n - rhead) / 4 / ftk::kWave;
+        if (rtiles == 0 || rtiles > 0x7fffffffu) return scalar_part(0, n);
+        ftk::AdamArgs a;
+        a.p = p + rhead;
+        a.g = gb + rhead * gsz;
+        a.m = m + rhead;
+        a.v = v + rhead;
+        a.p_out = out.p + rhead;
+        a.m_out = out.m + rhead;
+        a.v_out = out.v + rhead;
+        a.h = h ? hb + rhead * 2 : nullptr;
+        a.ctl = ctl;
+        a.hyper = hyper;
+        a.n = rtiles * ftk::kWave;
+        a.c = c;
+        const unsigned lds = throttle_lds_bytes(48 + 4 * static_cast<unsigned>(gsz));
+        if (ctl)
+            hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, true>), dim3(static_cast<unsigned>(rtiles)), dim3(ftk::kWave),
+                               lds, stream, a, static_cast<uint64_t>(0));
+        else
+            hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, false>), dim3(static_cast<unsigned>(rtiles)), dim3(ftk::kWave),
+                               lds, stream, a, static_cast<uint64_t>(0));
+        FT_HIP(hipGetLastError());
+        const size_t rbody = rtiles * ftk::kWave * 4;
+        int rc = scalar_part(0, rhead);
+        if (rc != FT_OK) return rc;
+        return scalar_part(rhead + rbody, n - rhead - rbody);
+    }
 
     // An in-place segment with edge elements is one launch of the many-segment kernel (tiles and
     // edges in the same grid) instead of up to three.
@@ -669,8 +701,8 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
         const size_t body_tiles = (sg.n - head) / (ftk::kWave * 4);
         const bool edge = head + (sg.n - head) % (ftk::kWave * 4) > 0;
         if (!vec_ok || body_tiles + 1 >= ftk::kMultiMaxWorkgroups) {
-            // arrays whose alignments disagree (element by element), or a segment too long for one
-            // grid: the single-segment path takes it
+            // arrays whose alignments disagree, or a segment too long for one grid: the
+            // single-segment path takes it
             rc = fth::launch_adam(c, p, sg.g, g_dtype, static_cast<float*>(sg.m), static_cast<float*>(sg.v), sg.half_out,
                                   half_dtype, sg.n, ctl, stream, nullptr, nullptr, nullptr,
                                   static_cast<const ftk::AdamConsts*>(sg.hyper));

@@ -225,6 +225,60 @@ __global__ __launch_bounds__(kWave) void adam_tile_kernel(AdamArgs a, uint64_t t
     }
 }
 
+// The update over whole tiles for arrays whose alignments disagree (a 16-bit copy cut at an odd
+// element, a state array one element off): the same tile shape, but every array is accessed through
+// vector types that promise only the alignment of one element, so the compiler emits whatever the
+// hardware takes at that alignment (whole 16-byte accesses at dword alignment, split ones below it),
+// with non-temporal global loads and stores. Slower than the aligned kernel (stores no longer cover
+// whole cache lines), far faster than one element per lane. The scalars may come from a.hyper.
+typedef float f32x4_e __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint16_t u16x4_e __attribute__((ext_vector_type(4), aligned(2)));
+
+template <int GT, int HT, bool HAS_CTL>
+__global__ __launch_bounds__(kWave) void adam_tile_relaxed_kernel(AdamArgs a, uint64_t tile0)
+{
+    AdamConsts c = a.c;
+    if (a.hyper) c = *a.hyper;
+    const uint64_t i = (tile0 + blockIdx.x) * kWave + threadIdx.x;  // this lane's 4-element unit
+    const bool out_of_place = a.p_out != a.p || a.m_out != a.m || a.v_out != a.v;
+    if constexpr (HAS_CTL) {
+        if (a.ctl->skip && !out_of_place) return;
+        c.grad_mult = a.ctl->grad_mult;
+    }
+    f32x4 p = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.p) + i);
+    f32x4 m = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.m) + i);
+    f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.v) + i);
+    bool skip = false;
+    if constexpr (HAS_CTL) skip = a.ctl->skip != 0;  // out of place: the old state still has to reach the outputs
+    if (!skip) {
+        f32x4 g;
+        if constexpr (GT == FT_F32) {
+            g = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.g) + i);
+        } else {
+            const u16x4_e w = __builtin_nontemporal_load(reinterpret_cast<const u16x4_e*>(a.g) + i);
+            g.x = half_to_float<GT>(w.x);
+            g.y = half_to_float<GT>(w.y);
+            g.z = half_to_float<GT>(w.z);
+            g.w = half_to_float<GT>(w.w);
+        }
+        adam_unit(p, g, m, v, c);
+    }
+    __builtin_nontemporal_store(static_cast<f32x4_e>(p), reinterpret_cast<f32x4_e*>(a.p_out) + i);
+    __builtin_nontemporal_store(static_cast<f32x4_e>(m), reinterpret_cast<f32x4_e*>(a.m_out) + i);
+    __builtin_nontemporal_store(static_cast<f32x4_e>(v), reinterpret_cast<f32x4_e*>(a.v_out) + i);
+    if constexpr (HT == FT_F16 || HT == FT_BF16) {
+        if (!skip) {
+            const uint32_t lo = pack2<HT>(p.x, p.y), hi = pack2<HT>(p.z, p.w);
+            u16x4_e w;
+            w.x = (uint16_t)(lo & 0xffffu);
+            w.y = (uint16_t)(lo >> 16);
+            w.z = (uint16_t)(hi & 0xffffu);
+            w.w = (uint16_t)(hi >> 16);
+            __builtin_nontemporal_store(w, reinterpret_cast<u16x4_e*>(a.h) + i);
+        }
+    }
+}
+
 // Element-at-a-time kernel for heads, tails and arrays whose alignments disagree. a.n counts
 // elements. Same arithmetic, so the result of an element never depends on which kernel took it.
 template <int GT, int HT>

@@ -124,8 +124,10 @@ def test_tails_and_offsets(cuda, oracle, n, offset):
         assert torch.equal(now[:offset], was[:offset]) and torch.equal(now[offset + n:], was[offset + n:])
 
 
-def test_mismatched_alignment_falls_back_to_scalar_kernel(cuda, oracle):
-    """Arrays whose element offsets differ cannot share a vector body; results must not change."""
+def test_mismatched_alignment_keeps_the_results(cuda, oracle):
+    """Arrays whose element offsets differ cannot share the aligned vector body (they go through the
+    tile kernel that assumes element alignment only, and its element-per-lane edges); results must
+    not change."""
     eng = _engine(**HP)
     n = 10_001
     P, G, M, V = _gen(n + 8, cuda, seed=9, g_dtype=torch.float16)
@@ -134,6 +136,44 @@ def test_mismatched_alignment_falls_back_to_scalar_kernel(cuda, oracle):
     want = _oracle_step(oracle, p, g, m, v, step=3, half_dtype=torch.float16)
     eng._step({"step": 3}, h, p, g, m, v)
     _compare("misaligned", (p, m, v, h), want, torch.float16)
+
+
+@pytest.mark.parametrize("odd_one,g_dtype,half_dtype", [
+    (odd, g, h) for g, h in ((torch.bfloat16, torch.bfloat16), (torch.float32, torch.float16), (torch.float16, None))
+    for odd in "pgmvh" if not (odd == "h" and h is None)])
+@pytest.mark.parametrize("control", [None, "scale", "skip"])
+def test_one_array_off_the_others(cuda, oracle, odd_one, g_dtype, half_dtype, control):
+    """One array starts 1, 2 or 3 elements into its buffer, the others at the start of theirs (a
+    16-bit copy cut at an odd element, a state array one element off): many tiles, bits as the
+    oracle's, nothing written outside the views, a skipped step leaves everything alone."""
+    eng = _engine(**HP)
+    n, pad = 300_003, 8
+    for shift in (1, 2, 3):
+        P, G, M, V = _gen(n + pad, cuda, seed=40 + shift, g_dtype=g_dtype)
+        H = torch.full((n + pad,), 7.0, dtype=half_dtype, device=cuda) if half_dtype is not None else None
+        offs = {k: (shift if k == odd_one else 0) for k in "pgmvh"}
+        p, g, m, v = (t[offs[k]:offs[k] + n] for k, t in (("p", P), ("g", G), ("m", M), ("v", V)))
+        h = H[offs["h"]:offs["h"] + n] if H is not None else None
+        before = {k: t.clone() for k, t in (("p", P), ("g", G), ("m", M), ("v", V), ("h", H)) if t is not None}
+        mult = 0.25 if control else 1.0
+        want = _oracle_step(oracle, p, g, m, v, step=9, half_dtype=half_dtype, grad_mult=mult)
+        kwargs = {}
+        if control:
+            rec = torch.zeros(4, dtype=torch.float32, device=cuda)
+            rec[1], rec[3] = mult, 1.0
+            rec.view(torch.int32)[0] = 1 if control == "skip" else 0
+            kwargs["control"] = rec
+        eng._step({"step": 9}, h, p, g, m, v, **kwargs)
+        if control == "skip":
+            for k, t in (("p", P), ("m", M), ("v", V), ("h", H)):
+                assert t is None or torch.equal(t, before[k]), (odd_one, shift, k)
+            continue
+        _compare(f"{odd_one} off by {shift}", (p, m, v, h), want, half_dtype)
+        for k, t in (("p", P), ("g", G), ("m", M), ("v", V), ("h", H)):
+            if t is not None:
+                o = offs[k]
+                assert torch.equal(t[:o], before[k][:o]) and torch.equal(t[o + n:], before[k][o + n:]), (odd_one, shift, k)
+        assert torch.equal(G, before["g"])
 
 
 def test_special_values(cuda, oracle):

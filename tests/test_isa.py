@@ -102,3 +102,16 @@ def test_many_segment_kernel_keeps_its_table_in_scalar_registers(kernels):
         assert len(re.findall(r"s_cselect_b32", body)) >= 15, name
         assert re.search(r"s_load_dwordx\d+ s\[\d+:\d+\], s\[\d+:\d+\], s\d+", body), name  # register offset: the computed record address
     assert seen == 3 * 3 * 2 * 2
+
+
+def test_relaxed_alignment_kernel_uses_full_width_accesses(kernels):
+    """Arrays whose alignments disagree are still moved 16 (8) bytes per lane and instruction."""
+    seen = 0
+    for name, body in kernels.items():
+        if "adam_tile_relaxed_kernel" not in name:
+            continue
+        seen += 1
+        assert len(re.findall(r"global_load_dwordx4 .* nt", body)) >= 3, name
+        assert len(re.findall(r"global_store_dwordx4 .* nt", body)) >= 3, name
+        assert not re.search(r"global_(load|store)_(ubyte|short|ushort)", body), name
+    assert seen == 3 * 3 * 2
