@@ -489,7 +489,7 @@ size_t accumulate_workspace_bytes(size_t n)
 }
 
 template <int AT, int GT, bool ZERO, bool STATS>
-int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, float scale, float pre_mult,
+int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, bool g_relaxed, float scale, float pre_mult,
                       ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, const Decide& dec, hipStream_t stream)
 {
     constexpr size_t asz = (AT == FT_F32) ? 4 : 2, gsz = (GT == FT_F32) ? 4 : 2;
@@ -514,7 +514,7 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
                            fth::throttle_lds_bytes(4 * static_cast<unsigned>(asz + gsz)), stream,
                            static_cast<void*>(static_cast<char*>(acc) + head * asz),
                            static_cast<void*>(static_cast<char*>(g) + head * gsz), static_cast<uint64_t>(nvec), scale,
-                           pre_mult, wave_parts, keep_from);
+                           pre_mult, wave_parts, keep_from, g_relaxed ? 1 : 0);
         FT_HIP(hipGetLastError());
         if (STATS) {
             reduce_blocks = waves < static_cast<size_t>(kReduceBlocks) ? static_cast<int>(waves) : kReduceBlocks;
@@ -537,23 +537,23 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, fl
 }
 
 template <int AT, int GT>
-int launch_accumulate_flags(bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec, float scale,
+int launch_accumulate_flags(bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec, bool g_relaxed, float scale,
                             float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, const Decide& dec, hipStream_t stream)
 {
-    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
-    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
-    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
-    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+    if (zero && stats) return launch_accumulate<AT, GT, true, true>(acc, g, n, head, nvec, g_relaxed, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+    if (zero) return launch_accumulate<AT, GT, true, false>(acc, g, n, head, nvec, g_relaxed, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+    if (stats) return launch_accumulate<AT, GT, false, true>(acc, g, n, head, nvec, g_relaxed, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+    return launch_accumulate<AT, GT, false, false>(acc, g, n, head, nvec, g_relaxed, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
 }
 
 template <int AT>
-int launch_accumulate_g(int g_dtype, bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec,
+int launch_accumulate_g(int g_dtype, bool zero, bool stats, void* acc, void* g, size_t n, size_t head, size_t nvec, bool g_relaxed,
                         float scale, float pre_mult, ftk::StatsPartial* parts, ft_grad_stats_t* stats_out, int stats_accumulate, const Decide& dec, hipStream_t stream)
 {
     switch (g_dtype) {
-        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
-        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
-        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+        case FT_F32: return launch_accumulate_flags<AT, FT_F32>(zero, stats, acc, g, n, head, nvec, g_relaxed, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+        case FT_F16: return launch_accumulate_flags<AT, FT_F16>(zero, stats, acc, g, n, head, nvec, g_relaxed, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
+        default: return launch_accumulate_flags<AT, FT_BF16>(zero, stats, acc, g, n, head, nvec, g_relaxed, scale, pre_mult, parts, stats_out, stats_accumulate, dec, stream);
     }
 }
 
@@ -864,12 +864,14 @@ int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t 
     if (n > 0 && (!acc || !g)) return fth::fail(FT_EINVAL, "acc and g must not be NULL");
     const size_t asz = elem_size(acc_dtype), gsz = elem_size(g_dtype);
     size_t head = 0, nvec = 0;
+    bool g_relaxed = false;
     if (n > 0) {
         if (!aligned(acc, asz) || !aligned(g, gsz)) return fth::fail(FT_EALIGN, "a pointer is not aligned to its element size");
         head = ((asz * 4 - (reinterpret_cast<uintptr_t>(acc) & (asz * 4 - 1))) & (asz * 4 - 1)) / asz;
         if (head > n) head = n;  // shorter than the way to the first boundary: edge elements only
-        if (head < n && !aligned(static_cast<char*>(g) + head * gsz, gsz * 4))
-            return fth::fail(FT_EALIGN, "acc and g must start at the same element offset modulo 4 of their buffers");
+        // g off its vector alignment where acc reaches its own: the kernel then reads (and clears) g
+        // through accesses that assume element alignment only
+        g_relaxed = head < n && !aligned(static_cast<char*>(g) + head * gsz, gsz * 4);
         // A long buffer: on to the first tile boundary of acc (256 elements = 1 KiB of fp32), so that
         // every tile's streaming stores cover whole cache lines (a multiple of 4 more: g stays aligned).
         if (n - head >= 16 * 256) {
@@ -890,9 +892,9 @@ int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t 
     }
     ft_grad_stats_t* out = static_cast<ft_grad_stats_t*>(stats_out);
     switch (acc_dtype) {
-        case FT_F32: return launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
-        case FT_F16: return launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
-        default: return launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
+        case FT_F32: return launch_accumulate_g<FT_F32>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, g_relaxed, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
+        case FT_F16: return launch_accumulate_g<FT_F16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, g_relaxed, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
+        default: return launch_accumulate_g<FT_BF16>(g_dtype, zero_g != 0, stats, acc, g, n, head, nvec, g_relaxed, scale, stats_pre_mult, parts, out, stats_accumulate, dec, stream);
     }
 }
 

@@ -680,7 +680,7 @@ __device__ __forceinline__ void stats_of_stored(float value, uint32_t bits, floa
 // descriptors cover only the units of this tile that exist, so lanes past nvec cannot store.
 template <int AT, int GT, bool ZERO, bool STATS>
 __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t tile, uint64_t nvec, float scale,
-                                                float pre_mult, float (&sums)[4], uint32_t& bad, bool keep)
+                                                float pre_mult, float (&sums)[4], uint32_t& bad, bool keep, bool g_relaxed)
 {
     constexpr uint32_t kAccUnit = (AT == FT_F32) ? 16 : 8, kGradUnit = (GT == FT_F32) ? 16 : 8;
     const uint64_t t0 = tile * 64;  // wave-uniform
@@ -689,7 +689,22 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
     const uint64_t i = t0 + threadIdx.x;
     if (threadIdx.x >= live) return;
 
-    const f32x4 g4 = load_g4<GT, true>(g, i);
+    // The gradient unit as raw bits, fetched either way before anything waits for it (g_relaxed: g
+    // does not reach its vector alignment where acc does, so element alignment only).
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    f32x4 g32;
+    u32x2 g16;
+    if constexpr (GT == FT_F32) {
+        if (!g_relaxed)
+            g32 = ld<true>(reinterpret_cast<const f32x4*>(g) + i);
+        else
+            g32 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(g) + i);
+    } else {
+        if (!g_relaxed)
+            g16 = ld<true>(reinterpret_cast<const u32x2*>(g) + i);
+        else
+            g16 = __builtin_bit_cast(u32x2, static_cast<u16x4>(__builtin_nontemporal_load(reinterpret_cast<const u16x4_e*>(g) + i)));
+    }
     f32x4 a4;
     if constexpr (AT == FT_F32) {
         a4 = ld<true>(reinterpret_cast<const f32x4*>(acc) + i);
@@ -699,6 +714,15 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
         a4.y = half_to_float<AT>(w.x >> 16);
         a4.z = half_to_float<AT>(w.y & 0xffffu);
         a4.w = half_to_float<AT>(w.y >> 16);
+    }
+    f32x4 g4;
+    if constexpr (GT == FT_F32) {
+        g4 = g32;
+    } else {
+        g4.x = half_to_float<GT>(g16.x & 0xffffu);
+        g4.y = half_to_float<GT>(g16.x >> 16);
+        g4.z = half_to_float<GT>(g16.y & 0xffffu);
+        g4.w = half_to_float<GT>(g16.y >> 16);
     }
     f32x4 r;
 #pragma unroll
@@ -734,6 +758,16 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
         }
     }
     if constexpr (ZERO) {
+        if (g_relaxed) {
+            if constexpr (GT == FT_F32) {
+                const f32x4_e z = {0.f, 0.f, 0.f, 0.f};
+                __builtin_nontemporal_store(z, reinterpret_cast<f32x4_e*>(g) + i);
+            } else {
+                const u16x4_e z = {0, 0, 0, 0};
+                __builtin_nontemporal_store(z, reinterpret_cast<u16x4_e*>(g) + i);
+            }
+            return;
+        }
         const __amdgpu_buffer_rsrc_t rg = tile_rsrc(static_cast<char*>(g) + t0 * kGradUnit, live * kGradUnit);
         if constexpr (GT == FT_F32) {
             const f32x4 z = {0.f, 0.f, 0.f, 0.f};
@@ -756,13 +790,13 @@ struct WavePartial {
 template <int AT, int GT, bool ZERO, bool STATS>
 __global__ __launch_bounds__(64) void grad_accumulate_kernel(void* acc, void* g, uint64_t nvec, float scale,
                                                              float pre_mult, WavePartial* __restrict__ wave_partials,
-                                                             uint64_t keep_from_tile)
+                                                             uint64_t keep_from_tile, int g_relaxed)
 {
     float sums[4] = {0.f, 0.f, 0.f, 0.f};
     uint32_t bad = 0;
     const uint64_t ntiles = (nvec + 63) / 64;
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x)
-        accumulate_tile<AT, GT, ZERO, STATS>(acc, g, tile, nvec, scale, pre_mult, sums, bad, tile >= keep_from_tile);
+        accumulate_tile<AT, GT, ZERO, STATS>(acc, g, tile, nvec, scale, pre_mult, sums, bad, tile >= keep_from_tile, g_relaxed != 0);
     if constexpr (STATS) {
         const float t = wave_sum((sums[0] + sums[1]) + (sums[2] + sums[3]));
         const uint32_t tb = wave_sum_u32(bad);

@@ -67,14 +67,34 @@ def test_fused_statistics_equal_a_separate_pass(cuda, oracle):
     assert d2.nonfinite == d.nonfinite and abs(d2.sumsq - d.sumsq) <= 2 * NORM_RTOL * d.sumsq
 
 
-def test_mismatched_element_offsets_are_refused(cuda):
+@pytest.mark.parametrize("acc_dtype,g_dtype", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.float16, torch.float16)])
+@pytest.mark.parametrize("zero", [False, True])
+def test_gradients_off_the_accumulators_alignment(cuda, oracle, acc_dtype, g_dtype, zero):
+    """acc and g cut at different element offsets of their buffers: g is then read (and cleared)
+    through accesses that assume element alignment only; the same bits, statistics included,
+    nothing outside the views touched. Lengths that differ are refused."""
     from flextrain_amd.loss_scaler import GradientGuard
     guard = GradientGuard(cuda)
-    a, g = torch.zeros(1000, device=cuda), torch.zeros(1001, device=cuda, dtype=torch.bfloat16)
-    with pytest.raises(ValueError, match="element offset"):
-        guard.accumulate(a, g[1:])
+    gen = torch.Generator(device=cuda).manual_seed(11)
+    n = 200_003
+    for a_off, g_off in ((0, 1), (2, 0), (3, 1), (1, 2), (0, 3)):
+        A = torch.randn(n + 8, device=cuda, generator=gen).to(acc_dtype)
+        G = (torch.randn(n + 8, device=cuda, generator=gen) * 0.1).to(g_dtype)
+        a, g = A[a_off:a_off + n], G[g_off:g_off + n]
+        an, gn = _bits(a).copy(), _bits(g).copy()
+        oracle.grad_accumulate(an, CODE[acc_dtype], gn, CODE[g_dtype], scale=0.5, zero_g=zero)
+        outside = (A[:a_off].clone(), A[a_off + n:].clone(), G[:g_off].clone(), G[g_off + n:].clone())
+        guard.begin()
+        guard.accumulate(a, g, scale=0.5, zero_grads=zero, with_stats=True)
+        d = guard.decide()
+        assert max_ulp_gpu(a, an) == 0, (a_off, g_off)
+        assert np.array_equal(_bits(g), gn)
+        assert torch.equal(A[:a_off], outside[0]) and torch.equal(A[a_off + n:], outside[1])
+        assert torch.equal(G[:g_off], outside[2]) and torch.equal(G[g_off + n:], outside[3])
+        bad, sumsq = oracle.grad_stats(an, CODE[acc_dtype])
+        assert d.nonfinite == bad == 0 and abs(d.sumsq - sumsq) <= 2 * NORM_RTOL * sumsq
     with pytest.raises(ValueError):
-        guard.accumulate(a, g)  # lengths differ
+        guard.accumulate(torch.zeros(1000, device=cuda), torch.zeros(1001, device=cuda, dtype=torch.bfloat16))  # lengths differ
 
 
 def test_accumulate_llama7b_layer(cuda, oracle):

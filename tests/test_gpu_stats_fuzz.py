@@ -61,12 +61,13 @@ def test_random_statistics_and_accumulation(cuda, oracle, seed):
         # fp16 gradients are kept small enough that an accumulator of any type stays finite unless a special value is planted
         G = (torch.randn(n + offset + 8, device=cuda, generator=gen) * 0.05 * min(loss_scale, 256.0)).to(g_dtype)
         A = (torch.randn(n + offset + 8, device=cuda, generator=gen) * 0.5).to(acc_dtype)
-        g, a = G[offset:offset + n], A[offset:offset + n]
+        g_offset = offset if rng.integers(0, 3) else int(rng.integers(0, 8))  # now and then g is cut elsewhere than acc
+        g, a = G[g_offset:g_offset + n], A[offset:offset + n]
         if rng.integers(0, 4) == 0:
             for _ in range(int(rng.integers(1, 4))):
                 g[int(rng.integers(0, n))] = SPECIALS[int(rng.integers(0, 3))]
         gn, an = _bits(g).copy(), _bits(a).copy()
-        outside = (A[:offset].clone(), A[offset + n:].clone(), G[:offset].clone(), G[offset + n:].clone())
+        outside = (A[:offset].clone(), A[offset + n:].clone(), G[:g_offset].clone(), G[g_offset + n:].clone())
         ws_ptr, ws_len = (ws.data_ptr(), ws_bytes) if workspace == "caller" else (None, 0)
         accumulate_flag = 1 if started else 0
         ctl_ptr = record.data_ptr() + 16
@@ -100,7 +101,7 @@ def test_random_statistics_and_accumulation(cuda, oracle, seed):
                 continue
             bad, sumsq = oracle.grad_stats(an, CODE[acc_dtype], pre_mult=inv)
         assert torch.equal(A[:offset], outside[0]) and torch.equal(A[offset + n:], outside[1]), (seed, call, "outside acc")
-        assert torch.equal(G[:offset], outside[2]) and torch.equal(G[offset + n:], outside[3]), (seed, call, "outside g")
+        assert torch.equal(G[:g_offset], outside[2]) and torch.equal(G[g_offset + n:], outside[3]), (seed, call, "outside g")
         bad_total, sumsq_total, started = bad_total + bad, sumsq_total + sumsq, True
         host = record.cpu()
         assert int(host[0:1].view(torch.int64).item()) == bad_total, (seed, call, kind, workspace)
