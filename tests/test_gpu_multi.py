@@ -184,8 +184,9 @@ def test_control_record_applies_to_every_segment(cuda, oracle):
 
 
 def test_segment_whose_arrays_disagree_in_alignment(cuda, oracle):
-    """Gradient cut at another element offset than the parameters: that segment goes element by
-    element through a launch of its own, its neighbours through the table."""
+    """Gradient cut at another element offset than the parameters: that segment goes through
+    launches of its own (the tile kernel that assumes element alignment only), its neighbours
+    through the table."""
     from flextrain_amd import FlexTrainCPUAdam
     from flextrain_amd.param_group import StepContext
     eng = FlexTrainCPUAdam(**BASE)
