@@ -456,7 +456,7 @@ struct Decide {
 
 // Statistics scratch of ft_grad_accumulate_static: block partials followed by one wavefront partial
 // per 256 elements, for calls of up to FT_STATIC_MAX_ELEMS elements. It is part of the loaded code
-// object, so every GPU the library runs on holds its own copy (8.1 MiB) until the process ends.
+// object, so every GPU the library runs on holds its own copy (16.1 MiB) until the process ends.
 // In host code the array's name is only a handle for hipGetSymbolAddress, never an address.
 constexpr size_t kStaticScratchBytes =
     sizeof(ftk::StatsPartial) * kMaxStatsBlocks + (static_cast<size_t>(FT_STATIC_MAX_ELEMS) / 256 + 1) * sizeof(ftk::WavePartial);

@@ -422,25 +422,6 @@ __global__ __launch_bounds__(kWave) void adam_multi_kernel(AdamMultiArgs a)
 // Sum across the 64 lanes of a wavefront with DPP lane permutes (no LDS): xor-1 and xor-2 inside
 // each quad, then mirror inside half rows and rows; every lane of a 16-lane row then holds the
 // row total, and the four row totals are read with v_readlane and added in a fixed order.
-__device__ __forceinline__ float wave_sum(float x)
-{
-    int xi;
-    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0xB1, 0xF, 0xF, false);  // quad_perm:[1,0,3,2]
-    x += __builtin_bit_cast(float, xi);
-    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x4E, 0xF, 0xF, false);  // quad_perm:[2,3,0,1]
-    x += __builtin_bit_cast(float, xi);
-    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x141, 0xF, 0xF, false);  // row_half_mirror
-    x += __builtin_bit_cast(float, xi);
-    xi = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x140, 0xF, 0xF, false);  // row_mirror
-    x += __builtin_bit_cast(float, xi);
-    const int b = __builtin_bit_cast(int, x);
-    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0));
-    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
-    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32));
-    const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
-    return (r0 + r1) + (r2 + r3);
-}
-
 __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t x)
 {
     x += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, 0xB1, 0xF, 0xF, false);
@@ -451,14 +432,50 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t x)
            (uint32_t)__builtin_amdgcn_readlane((int)x, 32) + (uint32_t)__builtin_amdgcn_readlane((int)x, 48);
 }
 
+// The same reduction for doubles: the two halves of every value travel through the same lane
+// permutes, the additions are fp64.
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double x)
+{
+    const uint64_t b = __builtin_bit_cast(uint64_t, x);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)b, CTRL, 0xF, 0xF, false);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(b >> 32), CTRL, 0xF, 0xF, false);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ double readlane_f64(double x, const int lane)
+{
+    const uint64_t b = __builtin_bit_cast(uint64_t, x);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), lane);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ double wave_sum_f64(double x)
+{
+    x += dpp_f64<0xB1>(x);   // quad_perm:[1,0,3,2]
+    x += dpp_f64<0x4E>(x);   // quad_perm:[2,3,0,1]
+    x += dpp_f64<0x141>(x);  // row_half_mirror
+    x += dpp_f64<0x140>(x);  // row_mirror
+    return (readlane_f64(x, 0) + readlane_f64(x, 16)) + (readlane_f64(x, 32) + readlane_f64(x, 48));
+}
+
+// x*x added to acc in fp64. The square of an fp32 value is exact in fp64 (24-bit significand), so
+// the only rounding is the addition's, and no finite fp32 value can make the sum overflow or vanish:
+// 3.4e38 squared is 1.2e77, 1.4e-45 squared 2e-90, both far inside the fp64 range.
+__device__ __forceinline__ double add_square(float x, double acc)
+{
+    const double d = (double)x;
+    return __builtin_fma(d, d, acc);
+}
+
 struct StatsPartial {
     double sumsq;
     uint64_t nonfinite;
 };
 
-// One 16-byte load = 8 sixteen-bit or 4 thirty-two-bit gradient elements.
+// One 16-byte load = 8 sixteen-bit or 4 thirty-two-bit gradient elements. Exact path: every element
+// is tested for inf/nan (exponent field all ones), counted if so, and squared in if not.
 template <int GT>
-__device__ __forceinline__ void stats_accumulate(u32x4 w, float pre_mult, float (&acc)[4], uint32_t& bad)
+__device__ __forceinline__ void stats_accumulate(u32x4 w, float pre_mult, double (&acc)[4], uint32_t& bad)
 {
     if constexpr (GT == FT_F32) {
         const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
@@ -467,7 +484,7 @@ __device__ __forceinline__ void stats_accumulate(u32x4 w, float pre_mult, float 
             const bool nf = (ws[k] & 0x7f800000u) == 0x7f800000u;
             const float x = __builtin_bit_cast(float, ws[k]) * pre_mult;
             bad += nf ? 1u : 0u;
-            acc[k] = __builtin_fmaf(nf ? 0.0f : x, nf ? 0.0f : x, acc[k]);
+            acc[k] = add_square(nf ? 0.0f : x, acc[k]);
         }
     } else {
         constexpr uint32_t kExp = (GT == FT_BF16) ? 0x7f80u : 0x7c00u;
@@ -479,8 +496,36 @@ __device__ __forceinline__ void stats_accumulate(u32x4 w, float pre_mult, float 
             const float xlo = half_to_float<GT>(lo) * pre_mult;
             const float xhi = half_to_float<GT>(hi) * pre_mult;
             bad += (nlo ? 1u : 0u) + (nhi ? 1u : 0u);
-            acc[k] = __builtin_fmaf(nlo ? 0.0f : xlo, nlo ? 0.0f : xlo, acc[k]);
-            acc[k] = __builtin_fmaf(nhi ? 0.0f : xhi, nhi ? 0.0f : xhi, acc[k]);
+            acc[k] = add_square(nlo ? 0.0f : xlo, acc[k]);
+            acc[k] = add_square(nhi ? 0.0f : xhi, acc[k]);
+        }
+    }
+}
+
+// Non-zero iff one of the elements of the load is inf or nan. For the 16-bit types both halves of a
+// word are tested at once: adding one unit of the exponent field's lowest bit to the masked field
+// carries into the sign position exactly when the field is all ones.
+template <int GT>
+__device__ __forceinline__ uint32_t nonfinite_marks(u32x4 w)
+{
+    constexpr uint32_t kField = (GT == FT_F32) ? 0x7f800000u : (GT == FT_BF16 ? 0x7f807f80u : 0x7c007c00u);
+    constexpr uint32_t kUnit = (GT == FT_F32) ? 0x00800000u : (GT == FT_BF16 ? 0x00800080u : 0x04000400u);
+    constexpr uint32_t kCarry = (GT == FT_F32) ? 0x80000000u : 0x80008000u;
+    return ((((w.x & kField) + kUnit) | ((w.y & kField) + kUnit)) | (((w.z & kField) + kUnit) | ((w.w & kField) + kUnit))) & kCarry;
+}
+
+// The same sums for a load that is known to hold finite elements only: no test, no select.
+template <int GT>
+__device__ __forceinline__ void stats_accumulate_finite(u32x4 w, float pre_mult, double (&acc)[4])
+{
+    const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        if constexpr (GT == FT_F32) {
+            acc[k] = add_square(__builtin_bit_cast(float, ws[k]) * pre_mult, acc[k]);
+        } else {
+            acc[k] = add_square(half_to_float<GT>(ws[k] & 0xffffu) * pre_mult, acc[k]);
+            acc[k] = add_square(half_to_float<GT>(ws[k] >> 16) * pre_mult, acc[k]);
         }
     }
 }
@@ -512,12 +557,10 @@ __device__ __forceinline__ void block_stats_epilogue(double lane_sum, uint32_t b
 
 // Stage 1: every block writes one StatsPartial. nvec = number of 16-byte units; the caller
 // handles the elements outside [0, nvec*per_unit) in grad_stats_final_kernel.
-// A lane adds squares in four fp32 accumulators and empties them into an fp64 sum every
-// kStatsFlushTiles tiles, so that no fp32 sum ever holds more than a few hundred terms however
-// many elements the call covers (with fp32 sums over the whole call the norm of 4e9 elements was
-// off by 3e-6).
-constexpr int kStatsFlushTiles = 16;
-
+// Every square is formed and added in fp64 (four accumulators per lane), in the vector body as in
+// the edges, so an element contributes the same whatever part of the call it falls into, and no
+// finite gradient can overflow the sum or vanish from it. A tile's loads are first screened for
+// inf/nan as a whole; only a lane that holds one takes the per-element path that counts and masks.
 // The gradients are read again by the update that follows the decision, so what of them still fits
 // the memory-side cache afterwards is worth keeping there: tiles from `keep_from_tile` on (the last
 // ones this pass touches) are read with ordinary loads, everything before with streaming loads that
@@ -530,10 +573,8 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
                                                            uint64_t keep_from_tile, const float* scale_dev)
 {
     if (scale_dev) pre_mult = *scale_dev;  // 1/loss_scale kept in device memory (wave-uniform load)
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    double lane_sum = 0.0;
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
     uint32_t bad = 0;
-    int pending = 0;
     constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
     const uint64_t ntiles = (nvec + kTile - 1) / kTile;
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
@@ -550,8 +591,16 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
                 for (int u = 0; u < UNROLL; ++u)
                     w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, 0);
             }
+            uint32_t marks = 0;
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(w[u], pre_mult, acc, bad);
+            for (int u = 0; u < UNROLL; ++u) marks |= nonfinite_marks<GT>(w[u]);
+            if (marks == 0) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) stats_accumulate_finite<GT>(w[u], pre_mult, acc);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(w[u], pre_mult, acc, bad);
+            }
         } else {
             for (int u = 0; u < UNROLL; ++u) {
                 const uint64_t i = base + (uint64_t)u * BLOCK;
@@ -559,14 +608,8 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
                 stats_accumulate<GT>(g[i], pre_mult, acc, bad);
             }
         }
-        if (++pending == kStatsFlushTiles) {
-            lane_sum += ((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3]);
-            acc[0] = acc[1] = acc[2] = acc[3] = 0.f;
-            pending = 0;
-        }
     }
-    lane_sum += ((double)acc[0] + (double)acc[1]) + ((double)acc[2] + (double)acc[3]);
-    block_stats_epilogue<BLOCK>(lane_sum, bad, partials);
+    block_stats_epilogue<BLOCK>((acc[0] + acc[1]) + (acc[2] + acc[3]), bad, partials);
 }
 
 // The per-step decision from a statistics record (one thread):
@@ -584,7 +627,9 @@ __device__ __forceinline__ void write_decision(uint64_t nonfinite, double sumsq,
     const float clip = (float)coef;
     ctl->skip = nonfinite != 0 ? 1u : 0u;
     ctl->grad_mult = clip * inv_scale;
-    ctl->grad_norm = (float)norm;
+    // the norm of finite fp32 gradients can exceed the fp32 range (two elements of 3e38): the
+    // informational copy saturates instead of turning into inf; clip is computed from the double
+    ctl->grad_norm = norm < 3.4028234663852886e38 ? (float)norm : 3.4028234663852886e38f;
     ctl->clip_coef = clip;
 }
 
@@ -652,8 +697,7 @@ __global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartia
             if (nf) {
                 b += 1;
             } else {
-                const float u = x * pre_mult;
-                s += (double)u * (double)u;
+                s = add_square(x * pre_mult, s);
             }
         }
         publish_stats(s, b, out, accumulate, inv_scale, max_norm, ctl);
@@ -666,13 +710,13 @@ __global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartia
 // (exactly what grad_stats_kernel would report for it), so that the pass over the gradients that
 // accumulation needs anyway also yields the overflow flag and the norm.
 template <int AT>
-__device__ __forceinline__ void stats_of_stored(float value, uint32_t bits, float pre_mult, float& acc, uint32_t& bad)
+__device__ __forceinline__ void stats_of_stored(float value, uint32_t bits, float pre_mult, double& acc, uint32_t& bad)
 {
     constexpr uint32_t kExp = (AT == FT_F32) ? 0x7f800000u : (AT == FT_BF16 ? 0x7f80u : 0x7c00u);
     const bool nf = (bits & kExp) == kExp;
     const float x = value * pre_mult;
     bad += nf ? 1u : 0u;
-    acc = __builtin_fmaf(nf ? 0.0f : x, nf ? 0.0f : x, acc);
+    acc = add_square(nf ? 0.0f : x, acc);
 }
 
 // One 64-unit tile: lane `threadIdx.x` takes unit tile*64 + lane when that is below nvec. All
@@ -680,7 +724,7 @@ __device__ __forceinline__ void stats_of_stored(float value, uint32_t bits, floa
 // descriptors cover only the units of this tile that exist, so lanes past nvec cannot store.
 template <int AT, int GT, bool ZERO, bool STATS>
 __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t tile, uint64_t nvec, float scale,
-                                                float pre_mult, float (&sums)[4], uint32_t& bad, bool keep, bool g_relaxed)
+                                                float pre_mult, double& sum, uint32_t& bad, bool keep, bool g_relaxed)
 {
     constexpr uint32_t kAccUnit = (AT == FT_F32) ? 16 : 8, kGradUnit = (GT == FT_F32) ? 16 : 8;
     const uint64_t t0 = tile * 64;  // wave-uniform
@@ -740,7 +784,7 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const float rk = r[k];  // a scalar copy: bit-casting the vector element itself reads lane 0
-                stats_of_stored<FT_F32>(rk, __builtin_bit_cast(uint32_t, rk), pre_mult, sums[k], bad);
+                stats_of_stored<FT_F32>(rk, __builtin_bit_cast(uint32_t, rk), pre_mult, sum, bad);
             }
         }
     } else {
@@ -754,7 +798,7 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
         if constexpr (STATS) {
             const uint32_t b[4] = {w.x & 0xffffu, w.x >> 16, w.y & 0xffffu, w.y >> 16};
 #pragma unroll
-            for (int k = 0; k < 4; ++k) stats_of_stored<AT>(half_to_float<AT>(b[k]), b[k], pre_mult, sums[k], bad);
+            for (int k = 0; k < 4; ++k) stats_of_stored<AT>(half_to_float<AT>(b[k]), b[k], pre_mult, sum, bad);
         }
     }
     if constexpr (ZERO) {
@@ -779,10 +823,12 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
     }
 }
 
-// What one wavefront-sized workgroup of the accumulation pass reports: 8 bytes per 256 elements.
+// What one wavefront-sized workgroup of the accumulation pass reports: 16 bytes per 256 elements.
+// The squares are formed and added in fp64 from the first element on (see add_square).
 struct WavePartial {
-    float sumsq;
+    double sumsq;
     uint32_t nonfinite;
+    uint32_t reserved;
 };
 
 // nvec = number of 4-element units; one 64-lane workgroup per 64 units (the loop only matters when
@@ -792,18 +838,19 @@ __global__ __launch_bounds__(64) void grad_accumulate_kernel(void* acc, void* g,
                                                              float pre_mult, WavePartial* __restrict__ wave_partials,
                                                              uint64_t keep_from_tile, int g_relaxed)
 {
-    float sums[4] = {0.f, 0.f, 0.f, 0.f};
+    double sum = 0.0;
     uint32_t bad = 0;
     const uint64_t ntiles = (nvec + 63) / 64;
     for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x)
-        accumulate_tile<AT, GT, ZERO, STATS>(acc, g, tile, nvec, scale, pre_mult, sums, bad, tile >= keep_from_tile, g_relaxed != 0);
+        accumulate_tile<AT, GT, ZERO, STATS>(acc, g, tile, nvec, scale, pre_mult, sum, bad, tile >= keep_from_tile, g_relaxed != 0);
     if constexpr (STATS) {
-        const float t = wave_sum((sums[0] + sums[1]) + (sums[2] + sums[3]));
+        const double t = wave_sum_f64(sum);
         const uint32_t tb = wave_sum_u32(bad);
         if (threadIdx.x == 0) {
             WavePartial w;
             w.sumsq = t;
             w.nonfinite = tb;
+            w.reserved = 0;
             wave_partials[blockIdx.x] = w;
         }
     }
@@ -825,7 +872,7 @@ __global__ __launch_bounds__(256) void reduce_wave_partials_kernel(const WavePar
     uint64_t b = 0;
     for (uint64_t i = lo + threadIdx.x; i < hi; i += 256) {
         const WavePartial w = wave_partials[i];
-        s += (double)w.sumsq;
+        s += w.sumsq;
         b += w.nonfinite;
     }
     s_sum[threadIdx.x] = s;
@@ -885,10 +932,8 @@ __global__ __launch_bounds__(256) void grad_accumulate_finish_kernel(void* acc, 
             stored = half_to_float<AT>(bits);
         }
         if constexpr (STATS) {
-            float one = 0.f;
             uint32_t nb = 0;
-            stats_of_stored<AT>(stored, bits, pre_mult, one, nb);
-            s += (double)one;
+            stats_of_stored<AT>(stored, bits, pre_mult, s, nb);
             b += nb;
         }
         if constexpr (ZERO) {

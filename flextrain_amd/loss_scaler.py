@@ -273,7 +273,7 @@ class GradientGuard:
         stats_ptr = self.stats_ptr if with_stats else None
         if with_stats:
             need = int(self._lib.ft_grad_accumulate_workspace_bytes(acc.numel()))
-            if need > self._ws_bytes:  # grows with the largest buffer seen (8 bytes per 256 elements)
+            if need > self._ws_bytes:  # grows with the largest buffer seen (16 bytes per 256 elements)
                 self._ws = torch.empty(need, dtype=torch.uint8, device=self.device)
                 self._ws_bytes = need
         inv_scale = float(1.0 / float(loss_scale))

@@ -46,6 +46,7 @@ typedef struct ft_step_control_t {
     uint32_t skip;   /* non-zero: leave p, m, v and the low-precision copy untouched    */
     float grad_mult; /* g32 = (float)g * grad_mult  (= clip_coef * 1/loss_scale)        */
     float grad_norm; /* L2 norm of the unscaled gradient, for the caller's information  */
+                     /* (saturates at FLT_MAX; the decision uses the fp64 value)        */
     float clip_coef; /* min(1, max_norm / (norm + 1e-6)), 1 when clipping is off        */
 } ft_step_control_t;
 
@@ -166,7 +167,7 @@ int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* ou
  * acc and g should start at the same element offset modulo 4 of their buffers (then both are moved
  * with aligned vector accesses); a g that does not is read and cleared through accesses that assume
  * element alignment only, with the same results. With statistics the
- * workspace must hold ft_grad_accumulate_workspace_bytes(n) bytes (8 bytes per 256 elements on
+ * workspace must hold ft_grad_accumulate_workspace_bytes(n) bytes (16 bytes per 256 elements on
  * top of the fixed part), or be NULL for the library's own buffer. */
 size_t ft_grad_accumulate_workspace_bytes(size_t n);
 int ft_grad_accumulate(void* acc, int acc_dtype, void* g, int g_dtype, size_t n, float scale, int zero_g,
@@ -193,7 +194,7 @@ int ft_grad_decide_dev(const void* g, int g_dtype, size_t n, const void* inv_sca
 /* ft_grad_accumulate_static: ft_grad_accumulate for callers that cannot allocate (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc). No counterpart in the
  * reference. Same arguments, results and kernels as ft_grad_accumulate, without the workspace: the
- * statistics scratch is a static device array inside the library (about 8.1 MiB on every GPU the
+ * statistics scratch is a static device array inside the library (about 16.1 MiB on every GPU the
  * library runs on, held until the process ends), so the call allocates and frees nothing, whatever
  * the size of earlier calls. At most FT_STATIC_MAX_ELEMS elements per call (FT_EINVAL beyond).
  * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two

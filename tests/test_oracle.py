@@ -470,6 +470,26 @@ def test_grad_stats_against_float64(oracle):
         assert bad == 2 and abs(sumsq - float((finite ** 2).sum())) <= 1e-12 * sumsq
 
 
+@pytest.mark.parametrize("code", [0, 2])
+def test_grad_stats_keeps_huge_and_tiny_finite_gradients(oracle, code):
+    """Finite gradients whose squares leave the fp32 range (|g| above 1.8e19 or below 1e-23) must
+    neither overflow the sum nor vanish from it: the sum is checked against exact rational
+    arithmetic, rounded to fp64 once, alone and mixed with ordinary values."""
+    from fractions import Fraction
+    for mags in ((1e-25,), (1e-20,), (1e19,), (1e20,), (3e38,), (1e-25, 3e-3, 1e-20), (1e19, -2.5, 3e38, 1e20, 1e-3)):
+        g32 = np.array(mags * 5, dtype=np.float32)
+        if code == 2:  # bf16 bit patterns of the same magnitudes (rounded to bf16)
+            t = torch.from_numpy(g32).to(torch.bfloat16)
+            g = t.view(torch.int16).numpy().view(np.uint16)
+            vals = t.to(torch.float32).numpy()
+        else:
+            g, vals = g32, g32
+        bad, sumsq = oracle.grad_stats(g, code)
+        exact = sum(Fraction(float(x)) ** 2 for x in vals)
+        assert bad == 0 and math.isfinite(sumsq) and sumsq > 0
+        assert abs(Fraction(sumsq) - exact) <= exact * Fraction(1, 10 ** 14), mags
+
+
 def test_clip_coefficient_and_multiplier(oracle):
     assert oracle.clip_coefficient(0.5, 1.0) == 1.0
     assert oracle.clip_coefficient(146.0, 1.0) == pytest.approx(1 / 146.000001)
