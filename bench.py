@@ -82,6 +82,33 @@ def _host_description():
     return {"cpu_model": model, "logical_cpus": os.cpu_count(), "numa_nodes": len(glob.glob("/sys/devices/system/node/node[0-9]*")) or 1}
 
 
+def _host_memory_limits():
+    """What bounds pinned host memory on this machine: installed and available memory, the
+    locked-memory limit of the process, and the memory limit of its control group (if any)."""
+    import resource
+    out = {}
+    try:
+        with open("/proc/meminfo") as f:
+            for line in f:
+                key, _, rest = line.partition(":")
+                if key in ("MemTotal", "MemAvailable"):
+                    out["mem_total_gb" if key == "MemTotal" else "mem_available_gb"] = round(int(rest.split()[0]) * 1024 / 1e9, 1)
+    except OSError:
+        pass
+    soft, hard = resource.getrlimit(resource.RLIMIT_MEMLOCK)
+    out["rlimit_memlock"] = {"soft": "unlimited" if soft == resource.RLIM_INFINITY else soft,
+                             "hard": "unlimited" if hard == resource.RLIM_INFINITY else hard}
+    for path in ("/sys/fs/cgroup/memory.max", "/sys/fs/cgroup/memory/memory.limit_in_bytes"):
+        try:
+            with open(path) as f:
+                text = f.read().strip()
+            out["cgroup_memory_limit_gb"] = text if not text.isdigit() else round(int(text) / 1e9, 1)
+            break
+        except OSError:
+            continue
+    return out
+
+
 def _device_description(torch, dev):
     """What the runtime says about the GPU the figures were measured on (the roofline's peak is the
     published 8 TB/s; the memory clock and bus width the driver reports are listed beside it)."""
@@ -189,7 +216,10 @@ def link_probe(torch):
     _C.check("ft_link_probe", _C.lib().ft_link_probe(1 << 30, 10, ctypes.byref(r)))
     out = {name: getattr(r, name) for name, _ in _C.LinkProbe._fields_}
     out["unidirectional_ceiling_gbps"] = max(r.h2d_copy, r.d2h_copy, r.h2d_kernel, r.d2h_kernel)
-    out["bidirectional_sum_measured_gbps"] = max(r.both_copy, r.both_kernel)
+    pairings = {"copies both ways": r.both_copy, "copy kernels both ways": r.both_kernel,
+                "copies in, copy kernel out": r.both_copy_in_kernel_out, "copy kernel in, copies out": r.both_kernel_in_copy_out}
+    out["bidirectional_sum_measured_gbps"] = max(pairings.values())
+    out["best_bidirectional_pairing"] = max(pairings, key=pairings.get)
     out["full_duplex_ceiling_gbps"] = 2 * out["unidirectional_ceiling_gbps"]
     return out
 
@@ -209,6 +239,7 @@ def measure_offload(args, torch, dev, layers, steps, warmup):
     # The whole state must be pinned (3 x 4 bytes per element). A machine that cannot pin that much
     # runs the largest whole-layer prefix that fits, and the record says which fraction that is.
     p = None
+    pin_attempts = []  # what hipHostMalloc granted and refused on the way: shows that the size is the machine's
     while p is None:
         n = layers * N_7B_LAYER + 2 * 4096 * 32000
         t0 = time.perf_counter()
@@ -216,7 +247,10 @@ def measure_offload(args, torch, dev, layers, steps, warmup):
             p, m, v = (pinned_empty(n, torch.float32) for _ in range(3))
             spare = pinned_empty(3 << 30, torch.uint8)  # room for the link probe's own pinned buffers
             del spare
-        except _C.FtError:
+            pin_attempts.append({"layers": layers, "pinned_gb": round(3 * n * 4 / 1e9, 1), "granted": True})
+        except _C.FtError as exc:
+            pin_attempts.append({"layers": layers, "pinned_gb": round(3 * n * 4 / 1e9, 1), "granted": False,
+                                 "error": str(exc)[:120]})
             p = m = v = None
             gc.collect()
             layers -= 1
@@ -266,13 +300,16 @@ def measure_offload(args, torch, dev, layers, steps, warmup):
         torch.cuda.synchronize()
         ok = ok and torch.equal(bp.cpu(), p[lo:hi]) and torch.equal(bm.cpu(), m[lo:hi]) and torch.equal(bv.cpu(), v[lo:hi]) \
             and torch.equal(bh, h[lo:hi])
-    sec = sum(walls) / len(walls)
+    # the reference's statistic for its own probes: mean of the 20th..80th percentile band
+    sec = percentile_mean(walls)
     one_way = n * 12 / sec / 1e9
     record = {
         "workload": f"cfg5: offloaded Llama-7B optimizer ({layers} of 32 layers + embedding + lm_head), "
                     "fp32 p/m/v in pinned host DRAM streamed in chunks, bf16 grads and copy on GPU",
         "elements": n, "fraction_of_full_7b": n / n_full, "chunk_elems": chunk, "slots": args.slots, "chunks": -(-n // chunk),
-        "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "elements_per_s": n / sec,
+        "steps": steps, "warmup": warmup, "ms_per_step": sec * 1e3, "ms_per_step_statistic": "20-80 percentile mean",
+        "step_ms": [round(w * 1e3, 2) for w in walls], "ms_per_step_mean": sum(walls) / len(walls) * 1e3,
+        "elements_per_s": n / sec,
         "bytes_each_way": n * 12, "achieved_each_way_gbps": one_way, "achieved_total_gbps": 2 * one_way,
         "device_time_ms": sum(devs) / len(devs) * 1e3,
         "link": link,
@@ -281,6 +318,8 @@ def measure_offload(args, torch, dev, layers, steps, warmup):
         # ratio, not a fraction of a ceiling; it sits at 1.00 and may exceed it by a per cent
         "ratio_to_bidirectional_probe": 2 * one_way / link["bidirectional_sum_measured_gbps"],
         "setup": {"pinned_alloc_s": t_alloc, "init_s": t_init, "pinned_gb": 3 * n * 4 / 1e9},
+        "host": dict(_host_memory_limits(), pin_attempts=pin_attempts,
+                     largest_pinned_total_granted_gb=round((3 * n * 4 + (3 << 30)) / 1e9, 1)),
         "streamed_equals_resident_on_probe_chunks": bool(ok),
     }
     del p, m, v, g, h, before
@@ -310,18 +349,19 @@ def bench_offload(args, torch, dev) -> int:
     return 0 if ok else 3
 
 
-def bench_accumulate(args, torch, dev) -> int:
+def measure_accumulate(torch, dev, steps, warmup, calibration_copy=False):
     """Gradient hand-off before the step: fp32 accumulator += bf16 micro-batch gradient over the
     7B-layer partition, clearing the source and gathering the overflow/norm statistics of the
-    result in the same pass. Algorithmic bytes: read 4 + 2, write 4 + 2 = 12 B/element."""
+    result in the same pass. Algorithmic bytes: read 4 + 2, write 4 + 2 = 12 B/element. Returns
+    {variant: {ms_avg, achieved_gbps, bytes_per_element, wall_ms_per_step}}."""
+    from flextrain_amd import synth
     from flextrain_amd.loss_scaler import GradientGuard
+    from flextrain_amd.memory import allocate_device_arrays
     n = N_7B_LAYER
     guard = GradientGuard(dev)
-    from flextrain_amd.memory import allocate_device_arrays
-    from flextrain_amd import synth
     acc, g = allocate_device_arrays([(n, torch.float32), (n, torch.bfloat16)], dev)
     synth.fill_(g, 0, 3, scale=1e-3)
-    if args.calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
+    if calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
         scratch = torch.empty_like(acc)
         for _ in range(3):
             scratch.copy_(acc)
@@ -335,10 +375,10 @@ def bench_accumulate(args, torch, dev) -> int:
     results = {}
     for name, kw in variants.items():
         nbytes = kw.pop("bytes")
-        for _ in range(args.warmup):
+        for _ in range(warmup):
             guard.begin()
             guard.accumulate(acc, g, **kw)
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for a, b in ev:
@@ -350,7 +390,15 @@ def bench_accumulate(args, torch, dev) -> int:
         wall = time.perf_counter() - t0
         ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
         results[name] = {"ms_avg": ms, "achieved_gbps": n * nbytes / (ms * 1e-3) / 1e9, "bytes_per_element": nbytes,
-                         "wall_ms_per_step": wall * 1e3 / args.steps}
+                         "wall_ms_per_step": wall * 1e3 / steps}
+    del acc, g
+    torch.cuda.empty_cache()
+    return results
+
+
+def bench_accumulate(args, torch, dev) -> int:
+    n = N_7B_LAYER
+    results = measure_accumulate(torch, dev, args.steps, args.warmup, args.calibration_copy)
     main = results["accumulate+clear+stats"]
     print(json.dumps({
         "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
@@ -568,19 +616,20 @@ def bench_pipeline_resident(args, torch, dev, Unit) -> int:
     return 0
 
 
-def bench_multi(args, torch, dev) -> int:
-    """The 7B-layer partition of cfg2 cut into --segments ragged contexts of two parameter groups
+def measure_multi(torch, dev, segments, steps, warmup, calibration_copy=False, variants=("one_launch", "per_context")):
+    """The 7B-layer partition of cfg2 cut into `segments` ragged contexts of two parameter groups
     (different weight decay and step count), the way a unit's share reaches the step engine when
     groups and buffer pieces cut it (flextrain/param_group.py:365-477): all contexts in one launch
-    (ft_adam_step_multi) against one call per context (the reference's loop, flextrain/optimizer.py:44-69)."""
+    (ft_adam_step_multi) against one call per context (the reference's loop, flextrain/optimizer.py:44-69).
+    Returns (results by variant, the contexts' lengths)."""
     import random
 
     from flextrain_amd import FlexTrainCPUAdam
     from flextrain_amd.param_group import StepContext
-    n, k = N_7B_LAYER, max(1, args.segments)
+    n, k = N_7B_LAYER, max(1, segments)
     eng = FlexTrainCPUAdam(**HP)
     p, g, m, v, h = make_inputs(torch, n, torch.bfloat16, 1e-3, dev)
-    if args.calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
+    if calibration_copy:  # a plain copy of known size, to scale the profiler's byte counters by
         scratch = torch.empty_like(p)
         for _ in range(3):
             scratch.copy_(p)
@@ -601,9 +650,11 @@ def bench_multi(args, torch, dev) -> int:
 
     results = {}
     for name, fn in (("one_launch", one_launch), ("per_context", per_context)):
-        for _ in range(args.warmup):
+        if name not in variants:
+            continue
+        for _ in range(warmup):
             fn()
-        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         host = 0.0
@@ -617,20 +668,29 @@ def bench_multi(args, torch, dev) -> int:
         wall = time.perf_counter() - t0
         ms = sum(a.elapsed_time(b) for a, b in ev) / len(ev)
         results[name] = {"ms_avg": ms, "achieved_gbps": n * 28 / (ms * 1e-3) / 1e9, "frac": n * 28 / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                         "wall_ms_per_step": wall * 1e3 / args.steps, "host_us_per_step": host * 1e6 / args.steps}
+                         "wall_ms_per_step": wall * 1e3 / steps, "host_us_per_step": host * 1e6 / steps}
+    lengths = [c.full_parameter.numel() for c in ctxs]
+    del ctxs, p, g, m, v, h
+    torch.cuda.empty_cache()
+    return results, lengths
+
+
+def bench_multi(args, torch, dev) -> int:
+    n = N_7B_LAYER
+    results, lengths = measure_multi(torch, dev, args.segments, args.steps, args.warmup, args.calibration_copy)
     main = results["one_launch"]
     print(json.dumps({
         "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
         "value": n / (main["wall_ms_per_step"] * 1e-3), "unit": "elements/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": main["wall_ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"multi: the cfg2 partition cut into {len(ctxs)} ragged contexts of two parameter groups, "
-                               "stepped by one launch (against one call per context)", "elements": n, "segments": len(ctxs),
-                   "shortest": min(c.full_parameter.numel() for c in ctxs), "longest": max(c.full_parameter.numel() for c in ctxs)},
+        "config": {"workload": f"multi: the cfg2 partition cut into {len(lengths)} ragged contexts of two parameter groups, "
+                               "stepped by one launch (against one call per context)", "elements": n, "segments": len(lengths),
+                   "shortest": min(lengths), "longest": max(lengths)},
         "roofline": {"bound": "hbm", "kernel": "adam_multi_kernel", "achieved": main["achieved_gbps"], "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": main["frac"],
-                     "traffic": MEASURED_TRAFFIC_BYTES["multi"] if len(ctxs) == 16 else None,
-                     "traffic_source": TRAFFIC_SOURCE["multi"] if len(ctxs) == 16 else None,
+                     "traffic": MEASURED_TRAFFIC_BYTES["multi"] if len(lengths) == 16 else None,
+                     "traffic_source": TRAFFIC_SOURCE["multi"] if len(lengths) == 16 else None,
                      "algorithmic_bytes_per_launch": n * 28,
                      "kernel_ms_avg": main["ms_avg"]},
         "variants": results,
@@ -695,6 +755,93 @@ def bench_resident7b(args, torch, dev) -> int:
     return 0
 
 
+def measure_resident(torch, dev, workload, steps, warmup, calibration_copy=False):
+    """cfg2 / cfg3 / cfg4 with everything resident in HBM: `warmup` untimed steps, then `steps` timed
+    ones with HIP events on the stream the kernels run on (torch's current stream), recorded inside
+    the timed region: one in front of the statistics pass (when the workload has one), one in front
+    of the update, one behind it."""
+    from flextrain_amd import FlexTrainCPUAdam
+    from flextrain_amd.loss_scaler import GradientGuard
+    eng = FlexTrainCPUAdam(**HP)
+    if workload == "cfg2":
+        n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.bfloat16, 100, 1.0, None
+        p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev)
+        name = "cfg2: Llama-7B decoder-layer partition resident in HBM, bf16 grads, AdamW t=100, bf16 copy-out"
+        stats_pass = False
+    elif workload == "cfg3":
+        n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.float16, 100, 65536.0, None
+        p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev, scale=scale)
+        name = "cfg3: 7B-layer partition, fp16 grads x65536, fused overflow check + unscale + AdamW (no overflow)"
+        stats_pass = True
+    else:
+        n, g_dtype, t_step, scale, max_norm = N_70B_LAYER, torch.bfloat16, 1000, 1.0, 1.0
+        p, g, m, v, h = make_inputs(torch, n, g_dtype, 5e-3, dev)
+        name = "cfg4: Llama-70B-shaped layer partition, bf16 grads, global-norm clip to 1.0 + AdamW t=1000"
+        stats_pass = True
+    guard = GradientGuard(dev) if stats_pass else None
+    group = {"step": t_step}
+
+    def one_step():
+        if guard is not None:
+            guard.begin()
+            ctl = guard.add_and_decide(g, loss_scale=scale, max_grad_norm=max_norm)
+            eng._step(group, h, p, g, m, v, control=ctl)
+        else:
+            eng._step(group, h, p, g, m, v)
+
+    if calibration_copy:
+        scratch = torch.empty_like(p)
+        for _ in range(3):
+            scratch.copy_(p)
+        torch.cuda.synchronize()
+        del scratch
+
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        if guard is not None:
+            ev[i][0].record()
+            guard.begin()
+            ctl = guard.add_and_decide(g, loss_scale=scale, max_grad_norm=max_norm)
+            ev[i][1].record()
+            eng._step(group, h, p, g, m, v, control=ctl)
+        else:  # no statistics pass: one event pair around the update is all there is to time
+            ev[i][1].record()
+            eng._step(group, h, p, g, m, v)
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    upd_ms = [e[1].elapsed_time(e[2]) for e in ev]
+    pre_ms = [e[0].elapsed_time(e[1]) for e in ev] if guard is not None else [0.0]
+    whole_ms = [e[0].elapsed_time(e[2]) for e in ev] if guard is not None else upd_ms
+    del p, g, m, v, h
+    torch.cuda.empty_cache()
+    return {"n": n, "name": name, "grad_dtype": str(g_dtype).replace("torch.", ""), "bytes_per_elem": 28,
+            "stats_pass": stats_pass, "ms_per_step": wall * 1e3 / steps, "steps": steps, "warmup": warmup,
+            "upd_ms": upd_ms, "upd_avg": sum(upd_ms) / len(upd_ms), "pre_avg": sum(pre_ms) / len(pre_ms),
+            "whole_avg": sum(whole_ms) / len(whole_ms)}
+
+
+def guarded_step_record(r):
+    """Compact record of a step with a statistics pass in front (cfg3, cfg4): the whole step between
+    the first and the last HIP event, its two parts, and the fraction of the HBM peak at the step's
+    30 algorithmic bytes per element (2 for the statistics read, 28 for the update)."""
+    n = r["n"]
+    whole = r["whole_avg"]
+    return {"workload": r["name"], "elements": n, "steps": r["steps"], "warmup": r["warmup"],
+            "ms_per_step": whole, "wall_ms_per_step": r["ms_per_step"],
+            "update_ms": r["upd_avg"], "update_frac": n * 28 / (r["upd_avg"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "stats_ms": r["pre_avg"], "stats_frac": n * 2 / (r["pre_avg"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "bytes_per_element": 30, "frac": n * 30 / (whole * 1e-3) / 1e9 / HBM_PEAK_GBPS}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -727,6 +874,8 @@ def main() -> int:
     ap.add_argument("--stats-keep-mib", type=int, default=None,
                     help="cfg3/cfg4: MiB at the end of the statistics pass read with caching loads (default: the library's 256)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-side-records", action="store_true",
+                    help="cfg2: leave out the short side measurements (cfg3_step, cfg4_step, accumulate, multi16; about 5 s)")
     ap.add_argument("--no-offload-record", action="store_true",
                     help="cfg2: leave out the offloaded-streaming sub-record (cfg5 on the largest pinnable prefix, about 12 s)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -743,8 +892,7 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
-    from flextrain_amd import FlexTrainCPUAdam, _C
-    from flextrain_amd.loss_scaler import GradientGuard
+    from flextrain_amd import _C
     if not os.path.exists(_C.LIB_PATH):  # nothing built in this tree yet
         from flextrain_amd.build import build_library
         build_library()
@@ -763,87 +911,25 @@ def main() -> int:
         return bench_resident7b(args, torch, dev)
     if args.workload == "multi":
         return bench_multi(args, torch, dev)
-    eng = FlexTrainCPUAdam(**HP)
-
-    if args.workload == "cfg2":
-        n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.bfloat16, 100, 1.0, None
-        p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev)
-        name = "cfg2: Llama-7B decoder-layer partition resident in HBM, bf16 grads, AdamW t=100, bf16 copy-out"
-        bytes_per_elem, stats_pass = 28, False
-    elif args.workload == "cfg3":
-        n, g_dtype, t_step, scale, max_norm = N_7B_LAYER, torch.float16, 100, 65536.0, None
-        p, g, m, v, h = make_inputs(torch, n, g_dtype, 1e-3, dev, scale=scale)
-        name = "cfg3: 7B-layer partition, fp16 grads x65536, fused overflow check + unscale + AdamW (no overflow)"
-        bytes_per_elem, stats_pass = 28, True
-    else:
-        n, g_dtype, t_step, scale, max_norm = N_70B_LAYER, torch.bfloat16, 1000, 1.0, 1.0
-        p, g, m, v, h = make_inputs(torch, n, g_dtype, 5e-3, dev)
-        name = "cfg4: Llama-70B-shaped layer partition, bf16 grads, global-norm clip to 1.0 + AdamW t=1000"
-        bytes_per_elem, stats_pass = 28, True
-
-    guard = GradientGuard(dev) if stats_pass else None
-    group = {"step": t_step}
-
-    def one_step():
-        if guard is not None:
-            guard.begin()
-            ctl = guard.add_and_decide(g, loss_scale=scale, max_grad_norm=max_norm)
-            eng._step(group, h, p, g, m, v, control=ctl)
-        else:
-            eng._step(group, h, p, g, m, v)
-
-    if args.calibration_copy:
-        scratch = torch.empty_like(p)
-        for _ in range(3):
-            scratch.copy_(p)
-        torch.cuda.synchronize()
-        del scratch
-
-    for _ in range(args.warmup):
-        one_step()
-    torch.cuda.synchronize()
-
-    # Per-launch HIP events on the stream the kernels run on (torch's current stream), recorded
-    # inside the timed region: ev[i][0] before the update kernel, ev[i][1] after it.
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        if guard is not None:
-            ev[i][0].record()
-            guard.begin()
-            ctl = guard.add_and_decide(g, loss_scale=scale, max_grad_norm=max_norm)
-            ev[i][1].record()
-            eng._step(group, h, p, g, m, v, control=ctl)
-        else:  # no statistics pass: one event pair around the update is all there is to time
-            ev[i][1].record()
-            eng._step(group, h, p, g, m, v)
-        ev[i][2].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    upd_ms = [e[1].elapsed_time(e[2]) for e in ev]
-    pre_ms = [e[0].elapsed_time(e[1]) for e in ev] if guard is not None else [0.0]
-    upd_avg = sum(upd_ms) / len(upd_ms)
-    ms_per_step = wall * 1e3 / args.steps
-    alg_bytes = n * bytes_per_elem
+    r = measure_resident(torch, dev, args.workload, args.steps, args.warmup, args.calibration_copy)
+    n, upd_ms, upd_avg = r["n"], r["upd_ms"], r["upd_avg"]
+    alg_bytes = n * r["bytes_per_elem"]
     achieved = alg_bytes / (upd_avg * 1e-3) / 1e9
     out = {
         "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
-        "value": n / (ms_per_step * 1e-3),
+        "value": n / (r["ms_per_step"] * 1e-3),
         "unit": "elements/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": r["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": name, "elements": n, "grad_dtype": str(g_dtype).replace("torch.", ""),
-                   "copy_dtype": "bfloat16", "bytes_per_element": bytes_per_elem},
+        "config": {"workload": r["name"], "elements": n, "grad_dtype": r["grad_dtype"],
+                   "copy_dtype": "bfloat16", "bytes_per_element": r["bytes_per_elem"]},
         "hbm_gbps": achieved,
         "hbm_frac_of_peak": achieved / HBM_PEAK_GBPS,
         "device": _device_description(torch, dev),
@@ -855,17 +941,34 @@ def main() -> int:
             "kernel_ms_p20_80": percentile_mean(upd_ms),
         },
     }
-    if stats_pass:
-        pre_avg = sum(pre_ms) / len(pre_ms)
-        out["stats_pass"] = {"kernel": "grad_stats_kernel", "ms_avg": pre_avg, "bytes": n * 2,
-                             "achieved_gbps": n * 2 / (pre_avg * 1e-3) / 1e9}
-    del p, g, m, v, h
-    torch.cuda.empty_cache()
+    if r["stats_pass"]:
+        out["stats_pass"] = {"kernel": "grad_stats_kernel", "ms_avg": r["pre_avg"], "bytes": n * 2,
+                             "achieved_gbps": n * 2 / (r["pre_avg"] * 1e-3) / 1e9}
+        out["guarded_step"] = guarded_step_record(r)
+    if args.workload == "cfg2" and not args.no_side_records:
+        # Every figure the documents quote, in front of whoever runs this file: the guarded steps of
+        # cfg3 and cfg4 (statistics pass + decision + update), the fused accumulation pass and the
+        # 16-context launch, each a short run of its own with the same harness as its --workload.
+        side_steps, side_warmup = min(args.steps, 20), min(args.warmup, 3)
+        for key, workload in (("cfg3_step", "cfg3"), ("cfg4_step", "cfg4")):
+            out[key] = guarded_step_record(measure_resident(torch, dev, workload, side_steps, side_warmup))
+        acc = measure_accumulate(torch, dev, side_steps, side_warmup)
+        out["accumulate"] = {
+            "workload": "fp32 accumulator += bf16 gradient on the 7B-layer partition",
+            **{key: {"ms": acc[name]["ms_avg"], "bytes_per_element": acc[name]["bytes_per_element"],
+                     "frac": acc[name]["achieved_gbps"] / HBM_PEAK_GBPS}
+               for key, name in (("plain", "accumulate"), ("with_clear", "accumulate+clear"),
+                                 ("with_clear_and_statistics", "accumulate+clear+stats"))}}
+        multi, lengths = measure_multi(torch, dev, 16, side_steps, side_warmup)
+        out["multi16"] = {"workload": "the cfg2 partition as 16 ragged contexts of two parameter groups",
+                          "one_launch_ms": multi["one_launch"]["ms_avg"], "frac": multi["one_launch"]["frac"],
+                          "one_call_per_context_ms": multi["per_context"]["ms_avg"], "bytes_per_element": 28,
+                          "shortest": min(lengths), "longest": max(lengths)}
     if args.workload == "cfg2" and not args.no_offload_record:
         # The path's second target rides along: the offloaded optimizer streamed over the host link
-        # (cfg5 at the largest size this machine pins), 1 warm-up + 3 steps, beside the link probe.
+        # (cfg5 at the largest size this machine pins), 2 warm-ups + 5 steps, beside the link probe.
         try:
-            out["offload"], ok = measure_offload(args, torch, dev, args.layers, steps=3, warmup=1)
+            out["offload"], ok = measure_offload(args, torch, dev, args.layers, steps=5, warmup=2)
             if not ok:
                 out["offload"]["error"] = "streamed and resident results differ on the probe chunks"
         except Exception as exc:  # the headline figure must not depend on how much this machine can pin

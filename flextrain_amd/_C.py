@@ -32,7 +32,8 @@ class AdamSegment(ctypes.Structure):
 class LinkProbe(ctypes.Structure):
     """Mirror of ``ft_link_probe_t`` (GB/s; ``both_*`` is the sum of the two directions)."""
 
-    _fields_ = [(name, c_double) for name in ("h2d_copy", "d2h_copy", "both_copy", "h2d_kernel", "d2h_kernel", "both_kernel")]
+    _fields_ = [(name, c_double) for name in ("h2d_copy", "d2h_copy", "both_copy", "h2d_kernel", "d2h_kernel", "both_kernel",
+                                              "both_copy_in_kernel_out", "both_kernel_in_copy_out")]
 
 
 EXPORTS = {
@@ -83,6 +84,8 @@ EXPORTS = {
     "ft_synth_fill_host": (c_int, [c_void_p, c_int, c_size_t, c_uint64, c_uint32, c_uint64, c_int, c_float]),
     "ft_set_launch_tuning": (c_int, [c_int, c_int]),
     "ft_set_cache_tuning": (c_int, [c_size_t]),
+    "ft_set_stats_launches": (c_int, [c_int]),
+    "ft_release_stream_scratch": (c_int, [c_void_p]),
 }
 
 

@@ -16,6 +16,7 @@
 #include <mutex>
 #include <type_traits>
 #include <unordered_map>
+#include <vector>
 
 #include "ft_internal.hpp"
 #include "ft_kernels.hpp"
@@ -44,18 +45,27 @@ thread_local std::string t_last_error;
 std::mutex g_mu;
 std::unordered_map<int, fth::AdamObject> g_adams;
 std::unordered_map<int, int> g_cu_count;      // device -> compute units
-struct OwnedScratch {
-    void* ptr = nullptr;
+// What the library keeps per (device, stream) for the statistics passes enqueued there: a scratch
+// buffer for callers that bring none (calls on different streams never share one) and a ticket
+// counter for the one-launch statistics pass. Calls on one stream run in order, so they may share
+// both. ft_release_stream_scratch gives them back.
+struct StreamState {
+    void* ptr = nullptr;  // library-owned scratch, grown on demand
     size_t bytes = 0;
+    int ticket_slot = -1; // index into the device's ticket pool, -1: none assigned (yet, or pool exhausted)
 };
-// (device, stream) -> library-owned statistics scratch: calls on different streams never share one
-std::map<std::pair<int, hipStream_t>, OwnedScratch> g_stats_ws;
+std::map<std::pair<int, hipStream_t>, StreamState> g_stream_state;
+constexpr int kTicketSlots = 1024;
+constexpr int kTicketStride = 16;  // counters 64 bytes apart: one cache line each
+std::unordered_map<int, std::vector<int>> g_free_ticket_slots;  // device -> slots not in use
 int g_adam_waves_per_cu = FT_ADAM_WAVES_PER_CU;
 std::unordered_map<int, int> g_lds_per_cu;   // device -> bytes of LDS per compute unit
 std::atomic<int> g_stats_blocks_per_cu{FT_STATS_BLOCKS_PER_CU};  // read without the lock
 // How many bytes at the end of a statistics pass are read with caching loads (the size of the
 // memory-side cache of MI355X: what can still be there when the update reads the gradients again).
 std::atomic<size_t> g_stats_keep_bytes{static_cast<size_t>(256) << 20};
+// The statistics pass as one launch (the last block takes the final sum) or as two.
+std::atomic<int> g_stats_one_launch{1};
 
 constexpr int kMaxStatsBlocks = 8192;
 
@@ -424,7 +434,7 @@ int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need
         int dev = 0;
         FT_HIP(hipGetDevice(&dev));
         std::lock_guard<std::mutex> lk(g_mu);
-        OwnedScratch& own = g_stats_ws[std::make_pair(dev, stream)];
+        StreamState& own = g_stream_state[std::make_pair(dev, stream)];
         if (own.bytes < need) {
             if (own.ptr) FT_HIP(hipFree(own.ptr));
             own.ptr = nullptr;
@@ -441,6 +451,47 @@ int resolve_stats_workspace(void* workspace, size_t workspace_bytes, size_t need
         parts = static_cast<ftk::StatsPartial*>(own.ptr);
     }
     *out = parts;
+    return FT_OK;
+}
+
+// Ticket counters of the one-launch statistics pass: part of the loaded code object, so zero when
+// the library is loaded, and every pass leaves its counter at zero again. In host code the array's
+// name is only a handle for hipGetSymbolAddress, never an address.
+static __device__ __align__(256) uint32_t g_ticket_pool[kTicketSlots * kTicketStride];
+std::unordered_map<int, uint32_t*> g_ticket_pool_ptr;  // device -> that device's copy of the pool
+
+// The ticket counter of (current device, stream), or nullptr when the pass has to take two launches:
+// a stream under graph capture (the recorded kernel would be replayed on whatever stream the graph is
+// launched on, beside eager passes that own this counter), or no counter left.
+int stream_ticket(hipStream_t stream, uint32_t** out)
+{
+    *out = nullptr;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+        (void)hipGetLastError();
+        return FT_OK;
+    }
+    if (capture != hipStreamCaptureStatusNone) return FT_OK;
+    int dev = 0;
+    FT_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto pool = g_ticket_pool_ptr.find(dev);
+    if (pool == g_ticket_pool_ptr.end()) {
+        void* ptr = nullptr;
+        FT_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_ticket_pool)));
+        if (!ptr) return fth::fail(FT_EHIP, "hipGetSymbolAddress returned a null address for the ticket counters");
+        pool = g_ticket_pool_ptr.emplace(dev, static_cast<uint32_t*>(ptr)).first;
+        std::vector<int>& free_slots = g_free_ticket_slots[dev];
+        for (int k = kTicketSlots - 1; k >= 0; --k) free_slots.push_back(k);
+    }
+    StreamState& st = g_stream_state[std::make_pair(dev, stream)];
+    if (st.ticket_slot < 0) {
+        std::vector<int>& free_slots = g_free_ticket_slots[dev];
+        if (free_slots.empty()) return FT_OK;
+        st.ticket_slot = free_slots.back();
+        free_slots.pop_back();
+    }
+    *out = pool->second + static_cast<size_t>(st.ticket_slot) * kTicketStride;
     return FT_OK;
 }
 
@@ -563,7 +614,7 @@ extern "C" {
 
 const char* ft_last_error(void) { return t_last_error.c_str(); }
 
-int ft_abi_version(void) { return 2; }
+int ft_abi_version(void) { return 3; }
 
 int ft_device_count(void)
 {
@@ -765,6 +816,17 @@ int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* 
     }
     const size_t nvec = (n - head) / per_unit;
     const size_t tail_begin = head + nvec * per_unit;
+    ftk::StatsFinalArgs fin;
+    fin.g = g;
+    fin.head = head;
+    fin.tail_begin = tail_begin;
+    fin.n = n;
+    fin.out = static_cast<ft_grad_stats_t*>(out);
+    fin.accumulate = accumulate;
+    fin.inv_scale = dec.inv_scale;
+    fin.max_norm = dec.max_norm;
+    fin.ctl = dec.ctl;
+    fin.ticket = nullptr;
     int blocks = 0;
     if (nvec > 0) {
         constexpr size_t kTile = static_cast<size_t>(FT_STATS_BLOCK) * FT_STATS_UNROLL;
@@ -773,38 +835,44 @@ int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* 
         if (cap > static_cast<size_t>(kMaxStatsBlocks)) cap = kMaxStatsBlocks;
         if (b > cap) b = cap;
         blocks = static_cast<int>(b);
+        // One launch where the stream has a ticket counter of its own: the block that delivers the
+        // last partial also takes the final sum (and the decision).
+        if (g_stats_one_launch.load()) {
+            int trc = stream_ticket(stream, &fin.ticket);
+            if (trc != FT_OK) return trc;
+        }
         const ftk::u32x4* gv = reinterpret_cast<const ftk::u32x4*>(static_cast<const char*>(g) + head * esz);
         const size_t ntiles = (nvec + kTile - 1) / kTile, keep_tiles = g_stats_keep_bytes.load() / (kTile * 16);
         const uint64_t keep_from = ntiles > keep_tiles ? ntiles - keep_tiles : 0;
         switch (g_dtype) {
             case FT_F32:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F32, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev, fin);
                 break;
             case FT_F16:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_F16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev, fin);
                 break;
             default:
                 hipLaunchKernelGGL((ftk::grad_stats_kernel<FT_BF16, FT_STATS_BLOCK, FT_STATS_UNROLL>), dim3(blocks),
-                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev);
+                                   dim3(FT_STATS_BLOCK), 0, stream, gv, nvec, pre_mult, parts, keep_from, dec.scale_dev, fin);
                 break;
         }
         FT_HIP(hipGetLastError());
+        if (fin.ticket) return FT_OK;
     }
-    ft_grad_stats_t* o = static_cast<ft_grad_stats_t*>(out);
     switch (g_dtype) {
         case FT_F32:
-            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl, dec.scale_dev);
+            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F32>), dim3(1), dim3(256), 0, stream, parts, blocks, pre_mult,
+                               dec.scale_dev, fin);
             break;
         case FT_F16:
-            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl, dec.scale_dev);
+            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_F16>), dim3(1), dim3(256), 0, stream, parts, blocks, pre_mult,
+                               dec.scale_dev, fin);
             break;
         default:
-            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_BF16>), dim3(1), dim3(256), 0, stream, parts, blocks, g,
-                               head, tail_begin, n, pre_mult, o, accumulate, dec.inv_scale, dec.max_norm, dec.ctl, dec.scale_dev);
+            hipLaunchKernelGGL((ftk::grad_stats_final_kernel<FT_BF16>), dim3(1), dim3(256), 0, stream, parts, blocks, pre_mult,
+                               dec.scale_dev, fin);
             break;
     }
     FT_HIP(hipGetLastError());
@@ -944,6 +1012,28 @@ int ft_grad_control(const void* stats, float inv_scale, float max_norm, void* ct
                        static_cast<const ft_grad_stats_t*>(stats), inv_scale, max_norm,
                        static_cast<ft_step_control_t*>(ctl_out));
     FT_HIP(hipGetLastError());
+    return FT_OK;
+}
+
+int ft_release_stream_scratch(void* stream_)
+{
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    int dev = 0;
+    FT_HIP(hipGetDevice(&dev));
+    FT_HIP(hipStreamSynchronize(stream));  // nothing enqueued there may still use the buffer or the counter
+    std::lock_guard<std::mutex> lk(g_mu);
+    auto it = g_stream_state.find(std::make_pair(dev, stream));
+    if (it == g_stream_state.end()) return FT_OK;
+    if (it->second.ptr) FT_HIP(hipFree(it->second.ptr));
+    if (it->second.ticket_slot >= 0) g_free_ticket_slots[dev].push_back(it->second.ticket_slot);
+    g_stream_state.erase(it);
+    return FT_OK;
+}
+
+int ft_set_stats_launches(int launches)
+{
+    if (launches != 1 && launches != 2) return fth::fail(FT_EINVAL, "a statistics pass takes 1 or 2 launches, not %d", launches);
+    g_stats_one_launch = launches == 1 ? 1 : 0;
     return FT_OK;
 }
 

@@ -530,10 +530,10 @@ __device__ __forceinline__ void stats_accumulate_finite(u32x4 w, float pre_mult,
     }
 }
 
-// Block-level end of a statistics pass: per-lane fp64 sums and counts -> one partial per block,
-// added in a fixed tree order through LDS.
+// Block-level end of a statistics pass: per-lane fp64 sums and counts -> the block's totals, added
+// in a fixed tree order through LDS; valid in thread 0.
 template <int BLOCK>
-__device__ __forceinline__ void block_stats_epilogue(double lane_sum, uint32_t bad, StatsPartial* __restrict__ partials)
+__device__ __forceinline__ void block_stats_reduce(double lane_sum, uint32_t bad, double& total, uint64_t& total_bad)
 {
     __shared__ double s_sum[BLOCK];
     __shared__ uint32_t s_bad[BLOCK / kWave];
@@ -546,70 +546,39 @@ __device__ __forceinline__ void block_stats_epilogue(double lane_sum, uint32_t b
         if ((int)threadIdx.x < w) s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
         __syncthreads();
     }
+    total = 0.0;
+    total_bad = 0;
     if (threadIdx.x == 0) {
         uint64_t b = 0;
 #pragma unroll
         for (int k = 0; k < BLOCK / kWave; ++k) b += s_bad[k];
-        partials[blockIdx.x].sumsq = s_sum[0];
-        partials[blockIdx.x].nonfinite = b;
+        total = s_sum[0];
+        total_bad = b;
     }
 }
 
-// Stage 1: every block writes one StatsPartial. nvec = number of 16-byte units; the caller
-// handles the elements outside [0, nvec*per_unit) in grad_stats_final_kernel.
-// Every square is formed and added in fp64 (four accumulators per lane), in the vector body as in
-// the edges, so an element contributes the same whatever part of the call it falls into, and no
-// finite gradient can overflow the sum or vanish from it. A tile's loads are first screened for
-// inf/nan as a whole; only a lane that holds one takes the per-element path that counts and masks.
-// The gradients are read again by the update that follows the decision, so what of them still fits
-// the memory-side cache afterwards is worth keeping there: tiles from `keep_from_tile` on (the last
-// ones this pass touches) are read with ordinary loads, everything before with streaming loads that
-// leave nothing behind. The update's own traffic is streaming, so the kept lines survive until it
-// reaches them. Measured on the 7B-layer partition (405 MB of fp16 gradients, 256 MB cache): the
-// update behind an all-streaming pass takes 0.838 ms, behind a caching pass 0.79 ms.
-template <int GT, int BLOCK, int UNROLL>
-__global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restrict__ g, uint64_t nvec,
-                                                           float pre_mult, StatsPartial* __restrict__ partials,
-                                                           uint64_t keep_from_tile, const float* scale_dev)
+// A block partial as it crosses from the block that made it to the block that adds them all up
+// inside one launch. The compute units of MI355X sit in eight dies with a second-level cache each; a
+// release fence at device scope would write back that whole cache once per block (measured: the
+// statistics pass went from 66 to 85 us). The partial is therefore stored and loaded with
+// device-scope atomic accesses (relaxed), which bypass the per-die caches by themselves: once such a
+// store has completed (s_waitcnt), every later device-scope access on the device sees it.
+__device__ __forceinline__ void publish_partial(StatsPartial* slot, double sum, uint64_t bad)
 {
-    if (scale_dev) pre_mult = *scale_dev;  // 1/loss_scale kept in device memory (wave-uniform load)
-    double acc[4] = {0.0, 0.0, 0.0, 0.0};
-    uint32_t bad = 0;
-    constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
-    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
-    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const uint64_t base = tile * kTile + threadIdx.x;
-        if ((tile + 1) * kTile <= nvec) {
-            u32x4 w[UNROLL];
-            if (tile < keep_from_tile) {
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) w[u] = __builtin_nontemporal_load(g + base + (uint64_t)u * BLOCK);
-            } else {  // buffer loads with the default cache policy: a distinct instruction, so the two paths stay two
-                const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(g + tile * kTile), 0,
-                                                                                   (int)(kTile * 16), kRawBufferFlags);
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u)
-                    w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, 0);
-            }
-            uint32_t marks = 0;
-#pragma unroll
-            for (int u = 0; u < UNROLL; ++u) marks |= nonfinite_marks<GT>(w[u]);
-            if (marks == 0) {
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) stats_accumulate_finite<GT>(w[u], pre_mult, acc);
-            } else {
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(w[u], pre_mult, acc, bad);
-            }
-        } else {
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint64_t i = base + (uint64_t)u * BLOCK;
-                if (i >= nvec) break;
-                stats_accumulate<GT>(g[i], pre_mult, acc, bad);
-            }
-        }
-    }
-    block_stats_epilogue<BLOCK>((acc[0] + acc[1]) + (acc[2] + acc[3]), bad, partials);
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(&slot->sumsq), __builtin_bit_cast(uint64_t, sum), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&slot->nonfinite, bad, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both stores have arrived before anything below is issued
+}
+template <bool COHERENT>
+__device__ __forceinline__ StatsPartial read_partial(const StatsPartial* slot)
+{
+    if constexpr (!COHERENT) return *slot;  // written by an earlier launch
+    StatsPartial r;
+    r.sumsq = __builtin_bit_cast(double, __hip_atomic_load(reinterpret_cast<const uint64_t*>(&slot->sumsq), __ATOMIC_RELAXED,
+                                                           __HIP_MEMORY_SCOPE_AGENT));
+    r.nonfinite = __hip_atomic_load(&slot->nonfinite, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return r;
 }
 
 // The per-step decision from a statistics record (one thread):
@@ -647,61 +616,163 @@ __device__ __forceinline__ void publish_stats(double s, uint64_t b, ft_grad_stat
     if (ctl) write_decision(b, s, inv_scale, max_norm, ctl);
 }
 
-// Stage 2 (one block of 256): adds the block partials in a fixed tree order, then the up to
-// `edge` elements before/after the vector body one by one, and writes or accumulates the result.
-template <int GT>
-__global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartial* __restrict__ partials,
-                                                               int nparts, const void* g, uint64_t head,
-                                                               uint64_t tail_begin, uint64_t n, float pre_mult,
-                                                               ft_grad_stats_t* out, int accumulate, float inv_scale,
-                                                               float max_norm, ft_step_control_t* ctl,
-                                                               const float* scale_dev)
+// What the end of a statistics pass needs beside the block partials: the elements outside the
+// vector body, where the result goes, and the decision to take from it (ctl == nullptr: none).
+struct StatsFinalArgs {
+    const void* g;        // the whole gradient buffer
+    uint64_t head;        // elements in front of the vector body
+    uint64_t tail_begin;  // first element behind it
+    uint64_t n;
+    ft_grad_stats_t* out;
+    int accumulate;
+    float inv_scale;
+    float max_norm;
+    ft_step_control_t* ctl;
+    uint32_t* ticket;     // one-launch mode: counts the blocks that have delivered their partial; nullptr: two launches
+};
+
+// End of a statistics pass, run by the first 256 threads of ONE block (all threads of the block must
+// call it): adds the block partials in a fixed tree order, then the elements before/after the vector
+// body one by one, and writes or accumulates the result. The order of the additions depends on
+// nparts only, not on which block runs it.
+template <int GT, bool COHERENT>
+__device__ __forceinline__ void stats_final_block(const StatsPartial* partials, int nparts, float pre_mult, const StatsFinalArgs& f)
 {
-    if (scale_dev) pre_mult = inv_scale = *scale_dev;
-    __shared__ double s_sum[256];
-    __shared__ uint64_t s_bad[256];
-    double s = 0.0;
-    uint64_t b = 0;
-    for (int i = threadIdx.x; i < nparts; i += 256) {
-        s += partials[i].sumsq;
-        b += partials[i].nonfinite;
+    __shared__ double s_fsum[256];
+    __shared__ uint64_t s_fbad[256];
+    if (threadIdx.x < 256) {
+        double s = 0.0;
+        uint64_t b = 0;
+        for (int i = threadIdx.x; i < nparts; i += 256) {
+            const StatsPartial part = read_partial<COHERENT>(partials + i);
+            s += part.sumsq;
+            b += part.nonfinite;
+        }
+        s_fsum[threadIdx.x] = s;
+        s_fbad[threadIdx.x] = b;
     }
-    s_sum[threadIdx.x] = s;
-    s_bad[threadIdx.x] = b;
     __syncthreads();
     for (int w = 128; w > 0; w >>= 1) {
         if ((int)threadIdx.x < w) {
-            s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
-            s_bad[threadIdx.x] += s_bad[threadIdx.x + w];
+            s_fsum[threadIdx.x] += s_fsum[threadIdx.x + w];
+            s_fbad[threadIdx.x] += s_fbad[threadIdx.x + w];
         }
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        s = s_sum[0];
-        b = s_bad[0];
-        for (uint64_t i = 0; i < n; ++i) {
-            if (i == head) i = tail_begin;  // skip the vector body
-            if (i >= n) break;
+        double s = s_fsum[0];
+        uint64_t b = s_fbad[0];
+        for (uint64_t i = 0; i < f.n; ++i) {
+            if (i == f.head) i = f.tail_begin;  // skip the vector body
+            if (i >= f.n) break;
             float x;
             bool nf;
             if constexpr (GT == FT_F32) {
-                const uint32_t w = reinterpret_cast<const uint32_t*>(g)[i];
+                const uint32_t w = reinterpret_cast<const uint32_t*>(f.g)[i];
                 nf = (w & 0x7f800000u) == 0x7f800000u;
                 x = __builtin_bit_cast(float, w);
             } else {
                 constexpr uint32_t kExp = (GT == FT_BF16) ? 0x7f80u : 0x7c00u;
-                const uint32_t w = reinterpret_cast<const uint16_t*>(g)[i];
+                const uint32_t w = reinterpret_cast<const uint16_t*>(f.g)[i];
                 nf = (w & kExp) == kExp;
                 x = half_to_float<GT>(w);
             }
-            if (nf) {
+            if (nf)
                 b += 1;
-            } else {
+            else
                 s = add_square(x * pre_mult, s);
+        }
+        publish_stats(s, b, f.out, f.accumulate, f.inv_scale, f.max_norm, f.ctl);
+    }
+}
+
+// Stage 1: every block writes one StatsPartial. nvec = number of 16-byte units; the caller
+// handles the elements outside [0, nvec*per_unit) in grad_stats_final_kernel.
+// Every square is formed and added in fp64 (four accumulators per lane), in the vector body as in
+// the edges, so an element contributes the same whatever part of the call it falls into, and no
+// finite gradient can overflow the sum or vanish from it. A tile's loads are first screened for
+// inf/nan as a whole; only a lane that holds one takes the per-element path that counts and masks.
+// The gradients are read again by the update that follows the decision, so what of them still fits
+// the memory-side cache afterwards is worth keeping there: tiles from `keep_from_tile` on (the last
+// ones this pass touches) are read with ordinary loads, everything before with streaming loads that
+// leave nothing behind. The update's own traffic is streaming, so the kept lines survive until it
+// reaches them. Measured on the 7B-layer partition (405 MB of fp16 gradients, 256 MB cache): the
+// update behind an all-streaming pass takes 0.838 ms, behind a caching pass 0.79 ms.
+template <int GT, int BLOCK, int UNROLL>
+__global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restrict__ g, uint64_t nvec,
+                                                           float pre_mult, StatsPartial* partials,
+                                                           uint64_t keep_from_tile, const float* scale_dev, StatsFinalArgs fin)
+{
+    static_assert(BLOCK >= 256, "the final sum is taken by the first 256 threads of a block");
+    if (scale_dev) pre_mult = fin.inv_scale = *scale_dev;  // 1/loss_scale kept in device memory (wave-uniform load)
+    double acc[4] = {0.0, 0.0, 0.0, 0.0};
+    uint32_t bad = 0;
+    constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
+    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
+    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const uint64_t base = tile * kTile + threadIdx.x;
+        if ((tile + 1) * kTile <= nvec) {
+            u32x4 w[UNROLL];
+            if (tile < keep_from_tile) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) w[u] = __builtin_nontemporal_load(g + base + (uint64_t)u * BLOCK);
+            } else {  // buffer loads with the default cache policy: a distinct instruction, so the two paths stay two
+                const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(g + tile * kTile), 0,
+                                                                                   (int)(kTile * 16), kRawBufferFlags);
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u)
+                    w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, 0);
+            }
+            uint32_t marks = 0;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) marks |= nonfinite_marks<GT>(w[u]);
+            if (marks == 0) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) stats_accumulate_finite<GT>(w[u], pre_mult, acc);
+            } else {
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(w[u], pre_mult, acc, bad);
+            }
+        } else {
+            for (int u = 0; u < UNROLL; ++u) {
+                const uint64_t i = base + (uint64_t)u * BLOCK;
+                if (i >= nvec) break;
+                stats_accumulate<GT>(g[i], pre_mult, acc, bad);
             }
         }
-        publish_stats(s, b, out, accumulate, inv_scale, max_norm, ctl);
     }
+    double total;
+    uint64_t total_bad;
+    block_stats_reduce<BLOCK>((acc[0] + acc[1]) + (acc[2] + acc[3]), bad, total, total_bad);
+    if (fin.ticket == nullptr) {  // two launches: grad_stats_final_kernel follows
+        if (threadIdx.x == 0) {
+            partials[blockIdx.x].sumsq = total;
+            partials[blockIdx.x].nonfinite = total_bad;
+        }
+        return;
+    }
+    // One launch: every block draws a ticket once its partial has arrived where the whole device
+    // sees it; the block that draws the last one adds the partials up, in the same fixed order as the
+    // separate launch would, and leaves the ticket counter at zero for the next pass on this stream.
+    __shared__ uint32_t s_last;
+    if (threadIdx.x == 0) {
+        publish_partial(partials + blockIdx.x, total, total_bad);
+        s_last = __hip_atomic_fetch_add(fin.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1 ? 1u : 0u;
+    }
+    __syncthreads();
+    if (s_last == 0) return;
+    stats_final_block<GT, true>(partials, (int)gridDim.x, pre_mult, fin);
+    if (threadIdx.x == 0) __hip_atomic_store(fin.ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// The end of a statistics pass as a launch of its own (one block of 256): for a pass whose vector
+// body is empty and for callers that may not share a ticket counter (a stream under graph capture).
+template <int GT>
+__global__ __launch_bounds__(256) void grad_stats_final_kernel(const StatsPartial* partials, int nparts, float pre_mult,
+                                                               const float* scale_dev, StatsFinalArgs fin)
+{
+    if (scale_dev) pre_mult = fin.inv_scale = *scale_dev;
+    stats_final_block<GT, false>(partials, nparts, pre_mult, fin);
 }
 
 // ---- gradient accumulation ---------------------------------------------------------------------

@@ -328,11 +328,13 @@ struct LinkProbe {
         return hipGetLastError();
     }
 
-    // GB/s (1e9 bytes/s) summed over the directions in `mask` (bit 0: H2D, bit 1: D2H): the better of
+    // GB/s (1e9 bytes/s) summed over the directions in `mask` (bit 0: H2D, bit 1: D2H), direction d
+    // carried by a copy kernel when kernel[d], by the runtime's copies otherwise: the better of
     // one and of two transfers in flight per direction (on this platform two in flight help a single
     // direction a little and hurt both directions at once a lot: 70 against 97 GB/s).
-    int measure(int mask, bool kernel, int iters, double* gbps)
+    int measure(int mask, bool kernel_h2d, bool kernel_d2h, int iters, double* gbps)
     {
+        const bool kernel[2] = {kernel_h2d, kernel_d2h};
         *gbps = 0.0;
         for (int lanes = 1; lanes <= kLanes; ++lanes)
             for (int timed = 0; timed < 2; ++timed) {  // the first pass warms up
@@ -341,7 +343,7 @@ struct LinkProbe {
                 for (int i = 0; i < reps; ++i)
                     for (int l = 0; l < lanes; ++l)
                         for (int d = 0; d < 2; ++d)
-                            if (mask & (1 << d)) FT_HIP(transfer(d, l, kernel));
+                            if (mask & (1 << d)) FT_HIP(transfer(d, l, kernel[d]));
                 for (int d = 0; d < 2; ++d)
                     for (int l = 0; l < kLanes; ++l) FT_HIP(hipStreamSynchronize(stream[d][l]));
                 const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
@@ -355,12 +357,15 @@ struct LinkProbe {
     int run(int iters, ft_link_probe_t* out)
     {
         int rc;
-        if ((rc = measure(1, false, iters, &out->h2d_copy)) != FT_OK) return rc;
-        if ((rc = measure(2, false, iters, &out->d2h_copy)) != FT_OK) return rc;
-        if ((rc = measure(3, false, iters, &out->both_copy)) != FT_OK) return rc;
-        if ((rc = measure(1, true, iters, &out->h2d_kernel)) != FT_OK) return rc;
-        if ((rc = measure(2, true, iters, &out->d2h_kernel)) != FT_OK) return rc;
-        return measure(3, true, iters, &out->both_kernel);
+        if ((rc = measure(1, false, false, iters, &out->h2d_copy)) != FT_OK) return rc;
+        if ((rc = measure(2, false, false, iters, &out->d2h_copy)) != FT_OK) return rc;
+        if ((rc = measure(3, false, false, iters, &out->both_copy)) != FT_OK) return rc;
+        if ((rc = measure(1, true, true, iters, &out->h2d_kernel)) != FT_OK) return rc;
+        if ((rc = measure(2, true, true, iters, &out->d2h_kernel)) != FT_OK) return rc;
+        if ((rc = measure(3, true, true, iters, &out->both_kernel)) != FT_OK) return rc;
+        // the two mixed pairings: one direction by the runtime's copies, the other by a copy kernel
+        if ((rc = measure(3, false, true, iters, &out->both_copy_in_kernel_out)) != FT_OK) return rc;
+        return measure(3, true, false, iters, &out->both_kernel_in_copy_out);
     }
 };
 
@@ -878,7 +883,12 @@ int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps)
     int rc = ft_link_probe(bytes, iters, &r);
     if (rc != FT_OK) return rc;
     const double copy[3] = {r.h2d_copy, r.d2h_copy, r.both_copy}, kernel[3] = {r.h2d_kernel, r.d2h_kernel, r.both_kernel};
-    *out_gbps = copy[direction] > kernel[direction] ? copy[direction] : kernel[direction];
+    double best = copy[direction] > kernel[direction] ? copy[direction] : kernel[direction];
+    if (direction == 2) {
+        if (r.both_copy_in_kernel_out > best) best = r.both_copy_in_kernel_out;
+        if (r.both_kernel_in_copy_out > best) best = r.both_kernel_in_copy_out;
+    }
+    *out_gbps = best;
     return FT_OK;
 }
 

@@ -151,10 +151,21 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
  * a call needs a larger one (so a NULL-workspace call may allocate and wait for the device; bring
  * a workspace, or use ft_grad_accumulate_static, where that is not acceptable). Calls on different
  * streams never share a library-owned buffer.
+ * The pass is ONE kernel launch: the block that delivers the last partial sum also adds them up (in
+ * an order that depends on the grid only) and takes the decision, if one is asked for. It counts
+ * blocks in a counter the library keeps per (device, stream) -- calls on one stream run in order and
+ * share it, calls on different streams never do. A stream under graph capture gets the two-launch
+ * form instead (a recorded launch may be replayed on any stream), with the same results bit for bit.
+ *
+ * ft_release_stream_scratch: gives back what the library keeps for `stream` on the current device
+ * (the scratch buffer of NULL-workspace calls, the block counter). Waits for the stream first. Call
+ * it before destroying a stream that made statistics calls; a stream that is simply used again
+ * gets a new buffer and counter on its next call.
  */
 size_t ft_grad_stats_workspace_bytes(void);
 int ft_grad_stats(const void* g, int g_dtype, size_t n, float pre_mult, void* out, int accumulate,
                   void* workspace, size_t workspace_bytes, void* stream);
+int ft_release_stream_scratch(void* stream);
 
 /* ft_grad_accumulate: acc[i] = fma((float)g[i], scale, acc[i]) rounded to acc's type, in place;
  * scale == 1 is the plain accumulation the reference performs after every micro-batch when
@@ -294,12 +305,15 @@ int ft_offload_elapsed_ms(void* handle, float* out_ms);
  * device memory), hardened into a ceiling: `bytes` are moved per direction and iteration, every
  * figure the better of one and of two transfers in flight, once with the runtime's copies (*_copy) and once with a copy
  * kernel that reads or writes the pinned memory itself (*_kernel), host-to-device alone,
- * device-to-host alone, and both at once (both_*: the SUM of the two directions). GB/s = 1e9 bytes/s.
- * ft_link_bandwidth returns the better of the two methods for one direction code
+ * device-to-host alone, and both at once (both_*: the SUM of the two directions), the latter also in
+ * the two mixed pairings (both_copy_in_kernel_out: the runtime's copies host-to-device while a copy
+ * kernel writes device-to-host; both_kernel_in_copy_out: the reverse). GB/s = 1e9 bytes/s.
+ * ft_link_bandwidth returns the best of the methods for one direction code
  * (0 = host-to-device, 1 = device-to-host, 2 = both at once, summed). */
 typedef struct ft_link_probe_t {
     double h2d_copy, d2h_copy, both_copy;
     double h2d_kernel, d2h_kernel, both_kernel;
+    double both_copy_in_kernel_out, both_kernel_in_copy_out; /* since ABI version 3 */
 } ft_link_probe_t;
 int ft_link_probe(size_t bytes, int iters, ft_link_probe_t* out);
 int ft_link_bandwidth(size_t bytes, int iters, int direction, double* out_gbps);
@@ -336,6 +350,9 @@ int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu);
  * the memory-side cache; everything before is read with streaming loads. Default 256 MiB (the
  * cache of MI355X); 0 = stream everything, SIZE_MAX = cache everything. Speed only. */
 int ft_set_cache_tuning(size_t stats_keep_bytes);
+/* launches: 1 (default) = the statistics pass as one kernel launch, 2 = the partial sums and the
+ * final sum as two launches (what a stream under graph capture always gets). Same results. */
+int ft_set_stats_launches(int launches);
 
 #ifdef __cplusplus
 }

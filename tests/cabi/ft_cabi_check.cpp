@@ -333,10 +333,12 @@ void link_probe()
 {
     ft_link_probe_t r;
     FT_OK_OR_DIE(ft_link_probe(64u << 20, 2, &r));
-    std::printf("link: copies %.1f / %.1f / %.1f GB/s, copy kernel %.1f / %.1f / %.1f GB/s (H2D / D2H / both)\n", r.h2d_copy, r.d2h_copy,
-                r.both_copy, r.h2d_kernel, r.d2h_kernel, r.both_kernel);
-    check(r.h2d_copy > 1 && r.d2h_copy > 1 && r.both_copy > 1 && r.h2d_kernel > 1 && r.d2h_kernel > 1 && r.both_kernel > 1,
-          "link probe: six figures, all positive");
+    std::printf("link: copies %.1f / %.1f / %.1f GB/s, copy kernel %.1f / %.1f / %.1f GB/s (H2D / D2H / both), "
+                "copies in + kernel out %.1f, kernel in + copies out %.1f\n", r.h2d_copy, r.d2h_copy,
+                r.both_copy, r.h2d_kernel, r.d2h_kernel, r.both_kernel, r.both_copy_in_kernel_out, r.both_kernel_in_copy_out);
+    check(r.h2d_copy > 1 && r.d2h_copy > 1 && r.both_copy > 1 && r.h2d_kernel > 1 && r.d2h_kernel > 1 && r.both_kernel > 1 &&
+              r.both_copy_in_kernel_out > 1 && r.both_kernel_in_copy_out > 1,
+          "link probe: eight figures, all positive");
 }
 
 void offloaded_step(hipStream_t stream)

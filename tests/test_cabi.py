@@ -39,7 +39,7 @@ def test_header_is_plain_c(tmp_path):
 def test_registry_and_errors_without_a_gpu():
     from flextrain_amd import _C
     lib = _C.lib()
-    assert lib.ft_abi_version() == 2
+    assert lib.ft_abi_version() == 3
     assert lib.ft_grad_stats_workspace_bytes() > 0
     assert lib.ft_adam_create(31337, 1e-3, 0.9, 0.999, 1e-8, 0.01, 1, 0) == 0
     # n == 0 is a no-op that never touches the device
