@@ -450,7 +450,7 @@ def bench_pipeline(args, torch, dev) -> int:
             coord.initialize(opt, flat, mb, offload=True,
                              unit_windows={"auto": None, "off": False}.get(args.windows, True),
                              window_write_through=args.windows == "write_through",
-                             resident_units=args.resident_units)
+                             resident_units=args.resident_units, alpha=args.alpha)
         except _C.FtError:
             coord = None
             del opt, flat, params
@@ -463,7 +463,22 @@ def bench_pipeline(args, torch, dev) -> int:
     share = n // mb
     link = link_probe(torch)
 
-    def iteration():
+    phase_s = {"forward": [], "backward": []}
+
+    def iteration(timed=False):
+        # the reference's order (flextrain/engine.py:353-399): forward pass (steps the forward shares
+        # of the previous iteration), update_states, backward pass (steps the backward shares)
+        t0 = time.perf_counter()
+        coord.warmup_forward_pipeline()
+        for u in range(units):
+            coord.pre_unit_forward(u)
+            for k in range(mb):
+                coord.post_micro_batch_forward(u, k)
+        if timed:
+            coord.synchronize()
+            torch.cuda.synchronize()
+            phase_s["forward"].append(time.perf_counter() - t0)
+        t1 = time.perf_counter()
         opt.update_states()
         for u in reversed(range(units)):
             buf = coord.pre_unit_backward(u)
@@ -471,6 +486,9 @@ def bench_pipeline(args, torch, dev) -> int:
                 buf[k * share:(k + 1) * share].copy_(grads[k * share:(k + 1) * share])
                 coord.post_micro_batch_backward(u, k)
         coord.clear_backward_pipeline()
+        if timed:
+            torch.cuda.synchronize()
+            phase_s["backward"].append(time.perf_counter() - t1)
 
     for _ in range(args.warmup):
         iteration()
@@ -478,13 +496,21 @@ def bench_pipeline(args, torch, dev) -> int:
     for _ in range(args.steps):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        iteration()
+        iteration(timed=True)
         torch.cuda.synchronize()
         walls.append(time.perf_counter() - t0)
     sec = sum(walls) / len(walls)
     total = units * n
-    streamed = (units - min(args.resident_units, units)) * n
+    streamed_units = units - min(args.resident_units, units)
+    streamed = streamed_units * n
     one_way = streamed * 12 / sec / 1e9
+    # how the link's work falls into the two passes: each pass moves its share of every streamed unit
+    fwd_numel = coord._mb_fwd_numel * mb
+    phases = {}
+    for name, numel in (("forward", fwd_numel), ("backward", n - fwd_numel)):
+        t = sum(phase_s[name]) / len(phase_s[name])
+        phases[name] = {"ms": t * 1e3, "elements_per_unit": numel, "bytes_each_way": streamed_units * numel * 12,
+                        "each_way_gbps": streamed_units * numel * 12 / t / 1e9 if numel else 0.0}
     print(json.dumps({
         "metric": "Adam step elements/s + achieved HBM GB/s (% peak) on 7B-layer partition",
         "value": total / sec, "unit": "elements/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -495,8 +521,9 @@ def bench_pipeline(args, torch, dev) -> int:
                    "elements": total, "units": units, "micro_batches": mb, "chunk_elems": args.chunk_elems,
                    "slots": args.slots, "unit_windows": args.windows, "window_piece_mi": args.window_piece_mi,
                    "resident_units": min(args.resident_units, units),
-                   "streamed_elements": streamed},
+                   "streamed_elements": streamed, "alpha": args.alpha},
         "iteration_ms": [w * 1e3 for w in walls],
+        "phases": phases,
         "link": dict(link, achieved_each_way_gbps=one_way, achieved_total_gbps=2 * one_way,
                      frac_of_unidirectional=one_way / link["unidirectional_ceiling_gbps"],
                      ratio_to_bidirectional_probe=2 * one_way / link["bidirectional_sum_measured_gbps"]),
@@ -605,8 +632,8 @@ def bench_pipeline_resident(args, torch, dev, Unit) -> int:
         "config": {"workload": f"pipeline, resident: coordinator schedule over {units} Llama-7B layers, {mb} shares per unit, "
                                "fp32 state, bf16 grads and parameters all in HBM",
                    "elements": total, "units": units, "micro_batches": mb, "bytes_per_element": 34,
-                   "shares_per_unit": len(coord._unit_step_ctxts[0]),
-                   "contexts_per_unit": sum(len(coord._unit_step_ctxts[0][k]) for k in range(len(coord._unit_step_ctxts[0]))),
+                   "shares_per_unit": len(coord.unit_step_contexts(0)),
+                   "contexts_per_unit": sum(len(part) for part in coord.unit_step_contexts(0)),
                    "step_stream": coord._step_stream is not None, "backward_tokens": tokens},
         "host_ms_per_iteration": sum(host) / len(host) * 1e3,
         **({"backward_arithmetic_ms": arithmetic_ms, "exposed_optimizer_ms": sec * 1e3 - arithmetic_ms} if tokens else {}),
@@ -855,6 +882,9 @@ def main() -> int:
     ap.add_argument("--chunk-elems", type=int, default=64 * 1024 * 1024, help="cfg5: elements per streamed chunk")
     ap.add_argument("--slots", type=int, default=3, help="cfg5: device buffer sets of the pipeline")
     ap.add_argument("--layers", type=int, default=32, help="cfg5: decoder layers (32 = the full 7B optimizer)")
+    ap.add_argument("--alpha", type=float, default=0.0,
+                    help="pipeline: share of every unit's step that runs during the next forward pass instead of during "
+                         "backward (the reference's split_ratio.alpha)")
     ap.add_argument("--resident-units", type=int, default=0,
                     help="pipeline: units whose fp32 state stays in HBM although the others are streamed from host memory")
     ap.add_argument("--layer-groups", action="store_true",

@@ -85,6 +85,9 @@ EXPORTS = {
     "ft_set_launch_tuning": (c_int, [c_int, c_int]),
     "ft_set_cache_tuning": (c_int, [c_size_t]),
     "ft_set_stats_launches": (c_int, [c_int]),
+    "ft_set_launch_limit": (c_int, [c_uint64]),
+    "ft_launch_pieces": (c_int, [c_uint64, c_uint64, POINTER(c_uint64), POINTER(c_uint64), c_int]),
+    "ft_segment_batches": (c_int, [POINTER(c_uint64), c_int, c_uint64, POINTER(c_int)]),
     "ft_release_stream_scratch": (c_int, [c_void_p]),
 }
 

@@ -47,18 +47,29 @@ class HyperRecord:
     hyper-parameter changes; outside any capture; it waits for the device first, so that a step still
     in flight reads the values it was enqueued with); ``sync()`` enqueues the 48-byte copy to the device
     on the current stream -- recorded into a graph, that copy re-reads the staging copy at every
-    replay, so a recorded step follows the group from iteration to iteration."""
+    replay, so a recorded step follows the group from iteration to iteration. A step that meets a
+    record changed since its last ``sync()`` calls ``sync()`` itself first (eager callers need not
+    think of it; a recorded region should still hold its own ``sync()``, since a replay runs no
+    Python)."""
 
     def __init__(self, engine: "FlexTrainCPUAdam", device: torch.device):
         self._engine = engine
         self.host = torch.zeros(12, dtype=torch.int32, pin_memory=True)
         self.dev = torch.zeros(12, dtype=torch.int32, device=device)
+        #: the staging copy has changed since it last went to the device: a step that finds the flag
+        #: set copies the record over first (``_step`` / ``_step_many``), so that no caller can
+        #: consume a record that was never, or not since its last change, brought to the device
+        self.dirty = True
 
-    def fill(self, group_args: Dict, grad_mult: float = 1.0) -> "HyperRecord":
+    def fill(self, group_args: Dict, grad_mult: float = 1.0, wait: bool = True) -> "HyperRecord":
+        """``wait=False``: the caller has already waited for the device since the last step was
+        enqueued (one wait for all the groups of an optimizer instead of one per group)."""
         assert STEP_KEY in group_args, f"Key '{STEP_KEY}' not found in parameter group arguments."
         # A step enqueued earlier (or a graph replay) may not have copied the staging values yet:
         # they may only change once that work is done.
-        torch.cuda.synchronize(self.dev.device)
+        if wait:
+            torch.cuda.synchronize(self.dev.device)
+        self.dirty = True
         self._engine._set_defaults_args(group_args)
         beta1, beta2 = group_args["betas"]
         _C.check("ft_adam_hyper_fill", self._engine._lib.ft_adam_hyper_fill(
@@ -69,6 +80,7 @@ class HyperRecord:
 
     def sync(self) -> "HyperRecord":
         self.dev.copy_(self.host, non_blocking=True)
+        self.dirty = False
         return self
 
 
@@ -220,6 +232,8 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             record = group_args.get(HYPER_KEY)
             with torch.cuda.device(full_parameter.device):
                 if record is not None:  # the scalars are read from device memory (see HyperRecord)
+                    if record.dirty:
+                        record.sync()
                     if grad_mult != 1.0:
                         raise ValueError("a group with device-resident scalars takes its multiplier from the record "
                                          "(HyperRecord.fill(group, grad_mult=...)) or from a control record")
@@ -306,6 +320,9 @@ class FlexTrainCPUAdam(FlexTrainCPUOptimizer):
             if record is not None:
                 if grad_mult != 1.0:
                     raise ValueError("a group with device-resident scalars takes its multiplier from the record or a control record")
+                if record.dirty:
+                    with torch.cuda.device(device):
+                        record.sync()
                 seg.hyper = record.dev.data_ptr()
         with torch.cuda.device(device):
             _C.check("ft_adam_step_multi", self._lib.ft_adam_step_multi(

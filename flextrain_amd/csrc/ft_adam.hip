@@ -20,6 +20,7 @@
 
 #include "ft_internal.hpp"
 #include "ft_kernels.hpp"
+#include "ft_launch_plan.hpp"
 
 // Launch shape of the update kernel, from sweeps on MI355X at 2e8 elements: one 64-lane wavefront
 // per workgroup, one 4-element unit per lane, one workgroup per tile, non-temporal loads, streaming
@@ -66,6 +67,15 @@ std::atomic<int> g_stats_blocks_per_cu{FT_STATS_BLOCKS_PER_CU};  // read without
 std::atomic<size_t> g_stats_keep_bytes{static_cast<size_t>(256) << 20};
 // The statistics pass as one launch (the last block takes the final sum) or as two.
 std::atomic<int> g_stats_one_launch{1};
+// Workgroups (of 64 lanes) one launch may hold: what the runtime allows, or less when a test asks for
+// many launches of a modest amount of work (ft_set_launch_limit).
+std::atomic<uint64_t> g_launch_limit{ftk::kMaxWorkgroupsPerLaunch};
+inline uint64_t launch_limit() { return g_launch_limit.load(); }
+inline uint64_t multi_launch_limit()
+{
+    const uint64_t l = launch_limit();
+    return l < ftk::kMultiMaxWorkgroups ? l : ftk::kMultiMaxWorkgroups;
+}
 
 constexpr int kMaxStatsBlocks = 8192;
 
@@ -239,7 +249,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         const size_t head4 = ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4;
         const size_t rhead = head4 < n ? head4 : n;
         const size_t rtiles = (n - rhead) / 4 / ftk::kWave;
-        if (rtiles == 0 || rtiles > 0x7fffffffu) return scalar_part(0, n);
+        if (rtiles == 0) return scalar_part(0, n);
         ftk::AdamArgs a;
         a.p = p + rhead;
         a.g = gb + rhead * gsz;
@@ -254,13 +264,16 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.n = rtiles * ftk::kWave;
         a.c = c;
         const unsigned lds = throttle_lds_bytes(48 + 4 * static_cast<unsigned>(gsz));
-        if (ctl)
-            hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, true>), dim3(static_cast<unsigned>(rtiles)), dim3(ftk::kWave),
-                               lds, stream, a, static_cast<uint64_t>(0));
-        else
-            hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, false>), dim3(static_cast<unsigned>(rtiles)), dim3(ftk::kWave),
-                               lds, stream, a, static_cast<uint64_t>(0));
-        FT_HIP(hipGetLastError());
+        uint64_t tile0 = 0, blocks = 0;
+        for (uint64_t piece = 0; plan_launch_piece(rtiles, launch_limit(), piece, &tile0, &blocks); ++piece) {
+            if (ctl)
+                hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, true>), dim3(static_cast<unsigned>(blocks)), dim3(ftk::kWave),
+                                   lds, stream, a, tile0);
+            else
+                hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, false>), dim3(static_cast<unsigned>(blocks)), dim3(ftk::kWave),
+                                   lds, stream, a, tile0);
+            FT_HIP(hipGetLastError());
+        }
         const size_t rbody = rtiles * ftk::kWave * 4;
         int rc = scalar_part(0, rhead);
         if (rc != FT_OK) return rc;
@@ -270,7 +283,7 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
     // An in-place segment with edge elements is one launch of the many-segment kernel (tiles and
     // edges in the same grid) instead of up to three.
     const bool in_place = out.p == p && out.m == m && out.v == v;
-    if (in_place && (head > 0 || head + body < n) && ntiles + 1 < ftk::kMultiMaxWorkgroups) {
+    if (in_place && (head > 0 || head + body < n) && ntiles + 1 <= multi_launch_limit()) {
         ftk::AdamMultiArgs ma;
         ma.first_wg[0] = 0;
         for (int k = 1; k < ftk::kMultiMaxSegments; ++k) ma.first_wg[k] = 0xffffffffu;
@@ -304,9 +317,9 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         a.n = ntiles * ftk::kWave;
         a.c = c;
         const unsigned lds = throttle_lds_bytes(48 + 4 * static_cast<unsigned>(gsz));
-        const size_t max_grid = 0x7fffffffu;  // one workgroup per tile; a larger count is split
-        for (size_t tile0 = 0; tile0 < ntiles; tile0 += max_grid) {
-            const size_t blocks = (ntiles - tile0 < max_grid) ? (ntiles - tile0) : max_grid;
+        // one workgroup per tile; more tiles than a launch may hold workgroups are cut into several
+        uint64_t tile0 = 0, blocks = 0;
+        for (uint64_t piece = 0; plan_launch_piece(ntiles, launch_limit(), piece, &tile0, &blocks); ++piece) {
             auto launch = [&](auto has_ctl, auto has_hyper) {
                 hipLaunchKernelGGL((ftk::adam_tile_kernel<GT, HT, decltype(has_ctl)::value, decltype(has_hyper)::value>),
                                    dim3(static_cast<unsigned>(blocks)), dim3(ftk::kWave), lds, stream, a,
@@ -548,8 +561,10 @@ int launch_accumulate(void* acc, void* g, size_t n, size_t head, size_t nvec, bo
     if (nvec > 0) {
         // Like the update: one tile per wavefront-sized workgroup, residency throttled through
         // dynamic LDS so that the bytes in flight per compute unit stay at the tuned level.
+        // (the kernel's workgroups stride over the tiles, so a grid capped at what one launch may
+        // hold still covers them all)
         size_t waves = (nvec + 63) / 64;
-        if (waves > 0x7fffffffu) waves = 0x7fffffffu;
+        if (waves > launch_limit()) waves = static_cast<size_t>(launch_limit());
         // A pass that ends in a decision is followed by the update, which reads the accumulator as
         // its gradients: the last stats_keep_bytes of it are stored with the default cache policy so
         // that the update finds them in the memory-side cache (everything else streams).
@@ -751,7 +766,7 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
                             (!hb || aligned(hb + head * 2, 8));
         const size_t body_tiles = (sg.n - head) / (ftk::kWave * 4);
         const bool edge = head + (sg.n - head) % (ftk::kWave * 4) > 0;
-        if (!vec_ok || body_tiles + 1 >= ftk::kMultiMaxWorkgroups) {
+        if (!vec_ok || body_tiles + 1 > multi_launch_limit()) {
             // arrays whose alignments disagree, or a segment too long for one grid: the
             // single-segment path takes it
             rc = fth::launch_adam(c, p, sg.g, g_dtype, static_cast<float*>(sg.m), static_cast<float*>(sg.v), sg.half_out,
@@ -762,7 +777,7 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
         }
         const int which = (sg.half_out ? 1 : 0) | (sg.hyper ? 2 : 0);
         const unsigned wgs = static_cast<unsigned>(body_tiles) + (edge ? 1u : 0u);
-        if (batch[which].count == ftk::kMultiMaxSegments || batch[which].workgroups + static_cast<size_t>(wgs) > ftk::kMultiMaxWorkgroups)
+        if (fth::segment_batch_is_full(batch[which].count, batch[which].workgroups, wgs, ftk::kMultiMaxSegments, multi_launch_limit()))
             if ((rc = flush(which)) != FT_OK) return rc;
         Batch& b = batch[which];
         ftk::AdamSegment& d = b.a.seg[b.count];
@@ -1028,6 +1043,32 @@ int ft_release_stream_scratch(void* stream_)
     if (it->second.ticket_slot >= 0) g_free_ticket_slots[dev].push_back(it->second.ticket_slot);
     g_stream_state.erase(it);
     return FT_OK;
+}
+
+int ft_set_launch_limit(uint64_t max_workgroups)
+{
+    if (max_workgroups > ftk::kMaxWorkgroupsPerLaunch)
+        return fth::fail(FT_EINVAL, "a launch holds at most %llu workgroups of 64 lanes",
+                         static_cast<unsigned long long>(ftk::kMaxWorkgroupsPerLaunch));
+    g_launch_limit = max_workgroups == 0 ? ftk::kMaxWorkgroupsPerLaunch : max_workgroups;
+    return FT_OK;
+}
+
+int ft_launch_pieces(uint64_t workgroups, uint64_t limit, uint64_t* first, uint64_t* count, int capacity)
+{
+    if (limit == 0) limit = g_launch_limit.load();
+    const uint64_t pieces = fth::launch_piece_count(workgroups, limit);
+    if (pieces > 0x7fffffffull) return fth::fail(FT_EINVAL, "more pieces than an int can count");
+    for (uint64_t k = 0; k < pieces && static_cast<int64_t>(k) < capacity; ++k)
+        if (!fth::plan_launch_piece(workgroups, limit, k, first + k, count + k)) return fth::fail(FT_EINVAL, "piece %llu missing", static_cast<unsigned long long>(k));
+    return static_cast<int>(pieces);
+}
+
+int ft_segment_batches(const uint64_t* workgroups, int n_segs, uint64_t limit, int* batch_of)
+{
+    if (n_segs < 0 || (n_segs > 0 && (!workgroups || !batch_of))) return fth::fail(FT_EINVAL, "bad arguments");
+    if (limit == 0) limit = multi_launch_limit();
+    return fth::plan_segment_batches(workgroups, n_segs, ftk::kMultiMaxSegments, limit, batch_of);
 }
 
 int ft_set_stats_launches(int launches)

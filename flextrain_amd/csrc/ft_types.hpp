@@ -49,10 +49,19 @@ struct AdamSegment {
     AdamConsts c;
 };
 
+// The HIP runtime refuses a launch whose gridDim.x * blockDim.x exceeds 2^32 - 1 work-items
+// (hipErrorInvalidConfiguration), so a grid of 64-lane workgroups holds at most (2^32 - 1) / 64 of
+// them; whatever needs more is cut into several launches (plan_launch_pieces in ft_launch_plan.hpp).
+constexpr uint64_t kMaxThreadsPerLaunch = 0xffffffffull;
+constexpr uint64_t kMaxWorkgroupsPerLaunch = kMaxThreadsPerLaunch / 64;  // 67,108,863 workgroups of one wavefront
+
 // The whole table travels in the kernel-argument segment (1.6 KB): no device allocation, no upload.
 // first_wg[s] = (number of workgroups that belong to the segments before s) << 4 | s; unused
-// entries hold 0xffffffff. A launch therefore has fewer than 2^28 workgroups.
-constexpr unsigned kMultiMaxWorkgroups = (1u << 28) - 1;
+// entries hold 0xffffffff: the encoding leaves room for 2^28 - 1 workgroups, the runtime's limit on a
+// launch for fewer.
+constexpr uint64_t kMultiEncodingWorkgroups = (1ull << 28) - 1;
+constexpr uint64_t kMultiMaxWorkgroups =
+    kMultiEncodingWorkgroups < kMaxWorkgroupsPerLaunch ? kMultiEncodingWorkgroups : kMaxWorkgroupsPerLaunch;
 struct AdamMultiArgs {
     uint32_t first_wg[kMultiMaxSegments];
     const ft_step_control_t* ctl;

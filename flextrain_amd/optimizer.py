@@ -394,7 +394,11 @@ class FlexTrainOptimizer:
 
     def update_states(self):
         """Advances ``group["step"]`` of every group (reference ``:265-272``)."""
+        if self.capturable:
+            # a step in flight (or a graph replay) must have read the staging copies before they change:
+            # one wait for all groups
+            torch.cuda.synchronize()
         for group in self.param_groups:
             group[STEP_KEY] = group.get(STEP_KEY, 0) + 1
-            if self.capturable:  # staging copy only: the step itself brings it to the device
-                group["hyper_record"].fill(group)
+            if self.capturable:  # staging copy only: whatever steps next brings it to the device first
+                group["hyper_record"].fill(group, wait=False)

@@ -350,6 +350,18 @@ int ft_set_launch_tuning(int adam_waves_per_cu, int stats_blocks_per_cu);
  * the memory-side cache; everything before is read with streaming loads. Default 256 MiB (the
  * cache of MI355X); 0 = stream everything, SIZE_MAX = cache everything. Speed only. */
 int ft_set_cache_tuning(size_t stats_keep_bytes);
+/* How work is cut into launches. The runtime refuses a launch of more than 2^32 - 1 work-items in
+ * x, i.e. more than 67,108,863 workgroups of the 64 lanes these kernels use; an update or an
+ * accumulation pass over more tiles than that (above about 1.7e10 elements) is cut into several
+ * launches, and so is a many-segment call whose segments need more workgroups together.
+ * ft_set_launch_limit lowers the limit (0 restores it), so that the cutting can be exercised with
+ * ordinary sizes; results never depend on it. ft_launch_pieces reports how `workgroups` workgroups
+ * are cut under `limit` (0 = the current one): first[k], count[k] for piece k, at most `capacity`
+ * of them; returns the number of pieces. ft_segment_batches reports which launch each of n_segs
+ * segments (workgroups[i] workgroups each) of a many-segment call falls into. Neither touches a GPU. */
+int ft_set_launch_limit(uint64_t max_workgroups);
+int ft_launch_pieces(uint64_t workgroups, uint64_t limit, uint64_t* first, uint64_t* count, int capacity);
+int ft_segment_batches(const uint64_t* workgroups, int n_segs, uint64_t limit, int* batch_of);
 /* launches: 1 (default) = the statistics pass as one kernel launch, 2 = the partial sums and the
  * final sum as two launches (what a stream under graph capture always gets). Same results. */
 int ft_set_stats_launches(int launches);
