@@ -221,6 +221,9 @@ def link_probe(torch):
     out["bidirectional_sum_measured_gbps"] = max(pairings.values())
     out["best_bidirectional_pairing"] = max(pairings, key=pairings.get)
     out["full_duplex_ceiling_gbps"] = 2 * out["unidirectional_ceiling_gbps"]
+    # What the platform carries when both directions run at once, whichever way they are driven
+    # (copies both ways, copy kernels both ways, either mix): the limit an offloaded step lives under.
+    out["platform_full_duplex_each_way_gbps"] = out["bidirectional_sum_measured_gbps"] / 2
     return out
 
 
@@ -317,6 +320,11 @@ def measure_offload(args, torch, dev, layers, steps, warmup):
         # two measurements of the same limit (the probe's both-directions run and this step): a
         # ratio, not a fraction of a ceiling; it sits at 1.00 and may exceed it by a per cent
         "ratio_to_bidirectional_probe": 2 * one_way / link["bidirectional_sum_measured_gbps"],
+        # The step moves both directions at once, so what bounds it is what the link carries both
+        # ways at once: no pairing of copy methods in the probe carries more than
+        # bidirectional_sum_measured_gbps, which is below twice the unidirectional ceiling.
+        "ceiling_basis": "both-ways probe",
+        "ceiling_each_way_gbps": link["platform_full_duplex_each_way_gbps"],
         "setup": {"pinned_alloc_s": t_alloc, "init_s": t_init, "pinned_gb": 3 * n * 4 / 1e9},
         "host": dict(_host_memory_limits(), pin_attempts=pin_attempts,
                      largest_pinned_total_granted_gb=round((3 * n * 4 + (3 << 30)) / 1e9, 1)),

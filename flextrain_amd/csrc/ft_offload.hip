@@ -512,6 +512,50 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     }
     const bool in_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_IN;
     const bool out_staged = mode == FT_OFFLOAD_STAGED || mode == FT_OFFLOAD_STAGED_OUT;
+
+    // Everything that can refuse the step is settled before anything is enqueued: what the update
+    // launches check per chunk (alignment of every array to its element size, of the records to 16
+    // bytes) and every allocation the step needs (larger slots for a long step, staging for
+    // host-resident gradients or copy). An error therefore leaves the handle as it was, with nothing
+    // of the step in flight.
+    auto misaligned = [](const void* ptr, size_t a) { return (reinterpret_cast<uintptr_t>(ptr) & (a - 1)) != 0; };
+    if (misaligned(host_p, 4) || misaligned(host_m, 4) || misaligned(host_v, 4) || misaligned(g, gsz) ||
+        (half_out && misaligned(half_out, 2)))
+        return fth::fail(FT_EALIGN, "a pointer is not aligned to its element size");
+    if (ctl && misaligned(ctl, 16)) return fth::fail(FT_EALIGN, "ft_step_control_t must be 16-byte aligned");
+    const bool stage_g = g_on_host && in_staged;
+    // With a control record the step may turn out to be a no-op, and a skipped kernel writes no
+    // low-precision copy: a staged copy-back would then carry whatever the slot held before. The
+    // kernel therefore writes a host-resident copy itself, over the link, and on a skip the host
+    // array keeps its contents. (p, m and v need no such care: a skipped kernel whose outputs are
+    // not its inputs copies the old state through.)
+    const bool stage_h = half_out && half_on_host && out_staged && !ctl;
+    if (!window && (in_staged || out_staged)) {
+        if ((n + e->chunk - 1) / e->chunk + kRampExtraChunks > kMaxChunksPerStep) {
+            const size_t mi = 1u << 20, full = kMaxChunksPerStep - kRampExtraChunks;
+            const size_t grown = ((n + full - 1) / full + mi - 1) / mi * mi;
+            if ((rc = resize_slots(e, grown)) != FT_OK) return rc;
+        }
+        if (!e->slots.back().v && (rc = resize_slots(e, e->chunk)) != FT_OK) return rc;
+        for (Slot& s : e->slots) {
+            if (stage_g && !s.g) {
+                const hipError_t err = hipMalloc(&s.g, e->chunk * 4);
+                if (err != hipSuccess) {
+                    (void)hipGetLastError();
+                    s.g = nullptr;
+                    return fth::fail(FT_ENOMEM, "hipMalloc(%zu) for the gradient staging failed: %s", e->chunk * 4, hipGetErrorString(err));
+                }
+            }
+            if (stage_h && !s.h) {
+                const hipError_t err = hipMalloc(&s.h, e->chunk * 2);
+                if (err != hipSuccess) {
+                    (void)hipGetLastError();
+                    s.h = nullptr;
+                    return fth::fail(FT_ENOMEM, "hipMalloc(%zu) for the copy's staging failed: %s", e->chunk * 2, hipGetErrorString(err));
+                }
+            }
+        }
+    }
     // The pipeline starts after the producer of g/ctl on the caller's stream ...
     // (a step that copies nothing in -- inside a window, or with the kernel reading host memory
     // itself -- leaves the H2D stream alone)
@@ -579,24 +623,7 @@ int ft_offload_step(void* handle, int id, uint64_t step, float lr, float beta1, 
     const char* gb = static_cast<const char*>(g);
     char* hb = static_cast<char*>(half_out);
 
-    const bool stage_g = g_on_host && in_staged;
-    // With a control record the step may turn out to be a no-op, and a skipped kernel writes no
-    // low-precision copy: a staged copy-back would then carry whatever the slot held before. The
-    // kernel therefore writes a host-resident copy itself, over the link, and on a skip the host
-    // array keeps its contents. (p, m and v need no such care: a skipped kernel whose outputs are
-    // not its inputs copies the old state through.)
-    const bool stage_h = half_out && half_on_host && out_staged && !ctl;
-    if ((in_staged || out_staged) && (n + e->chunk - 1) / e->chunk + kRampExtraChunks > kMaxChunksPerStep) {
-        const size_t mi = 1u << 20, full = kMaxChunksPerStep - kRampExtraChunks;
-        const size_t grown = ((n + full - 1) / full + mi - 1) / mi * mi;
-        if ((rc = resize_slots(e, grown)) != FT_OK) return rc;
-    }
-    if ((in_staged || out_staged) && !e->slots.back().v && (rc = resize_slots(e, e->chunk)) != FT_OK) return rc;
     const size_t chunk = e->chunk;
-    for (Slot& s : e->slots) {
-        if (stage_g && !s.g) FT_HIP(hipMalloc(&s.g, chunk * 4));
-        if (stage_h && !s.h) FT_HIP(hipMalloc(&s.h, chunk * 2));
-    }
 
     // Chunk sizes of this step. Every chunk but the last starts and ends on a multiple of 256
     // elements (whole tiles at 1 KiB boundaries) whenever the chunk size itself is one.

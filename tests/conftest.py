@@ -10,6 +10,7 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    config.addinivalue_line("markers", "perf: a speed floor on the GPU (leave out with -m 'gpu and not perf')")
 
 
 @pytest.fixture(scope="session", autouse=True)

@@ -167,6 +167,34 @@ def test_pageable_host_memory_is_refused(cuda):
         eng._step({"step": 1}, None, p, g, m, v)
 
 
+def test_a_refused_step_leaves_nothing_enqueued(cuda, oracle):
+    """Whatever can refuse a streamed step is checked before anything is enqueued: a gradient pointer
+    off its element alignment in a step of several chunks returns FT_EALIGN with the host state
+    untouched and the engine idle, and the next good step runs as if nothing had happened."""
+    from flextrain_amd import FlexTrainCPUAdam, _C
+    n, chunk = 300_000, 1 << 16
+    eng = FlexTrainCPUAdam(offload_chunk_elems=chunk, offload_mode=1, **HP)
+    p, m, v = _host_state(n, 41)
+    before = [t.clone() for t in (p, m, v)]
+    gbuf = (torch.randn(n + 8, device=cuda) * 1e-3).to(torch.bfloat16)
+    g = gbuf[:n]
+    engine = eng._offload_engine()
+    lib = _C.lib()
+    rc = lib.ft_offload_step(engine, eng.opt_id, 3, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, 1.0, p.data_ptr(), gbuf.data_ptr() + 1,
+                             _C.BF16, 0, m.data_ptr(), v.data_ptr(), None, _C.F16, 0, n, None, _C.current_stream_ptr())
+    assert rc == -2 and b"aligned" in lib.ft_last_error()
+    bad_ctl = torch.zeros(8, dtype=torch.float32, device=cuda)
+    rc = lib.ft_offload_step(engine, eng.opt_id, 3, 1e-4, 0.9, 0.999, 1e-8, 0.01, 1, 1.0, p.data_ptr(), g.data_ptr(),
+                             _C.BF16, 0, m.data_ptr(), v.data_ptr(), None, _C.F16, 0, n, bad_ctl.data_ptr() + 4, _C.current_stream_ptr())
+    assert rc == -2
+    eng.synchronize()
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip((p, m, v), before))
+    want = _oracle(oracle, p, g, m, v, 3, None)
+    eng._step({"step": 3}, None, p, g, m, v)
+    _assert_equal_bits("after refused steps", p, m, v, None, want, None)
+
+
 def test_link_probe_reports_sane_numbers(cuda):
     import ctypes
     from flextrain_amd import _C

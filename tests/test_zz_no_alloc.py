@@ -1,9 +1,13 @@
-"""The entry point that allocates nothing: ft_grad_accumulate_static against ft_grad_accumulate.
+"""The entry point that allocates nothing: ft_grad_accumulate_static against ft_grad_accumulate and
+against the CPU checker.
 
-Called through the C ABI (ctypes on libftadam.so). Same kernels behind both, so everything is
-compared bit for bit: the accumulator, the cleared gradients and the statistics record, on two
-calls in a row on one GPU, the second with a smaller input (the static scratch still holds the
-first call's partials then), plus the size limit and the allocation-free property.
+Called through the C ABI (ctypes on libftadam.so). Same kernels behind both entry points, so
+everything is compared bit for bit: the accumulator, the cleared gradients and the statistics
+record, on two calls in a row on one GPU, the second with a smaller input (the static scratch still
+holds the first call's partials then), plus the size limit and the allocation-free property. The
+accumulator is also compared bit for bit with the checker's, and the statistics with its fp64 sum
+(count exact, sum of squares within 1e-9 relative), so that the two entry points cannot be wrong
+together.
 """
 import ctypes
 
@@ -32,9 +36,13 @@ def _bits(t):
 
 
 @pytest.mark.parametrize("acc_dtype,g_dtype", [(torch.float32, torch.bfloat16), (torch.float16, torch.float16)])
-def test_static_scratch_entry_point_equals_the_workspace_one(cuda, acc_dtype, g_dtype):
+def test_static_scratch_entry_point_equals_the_workspace_one(cuda, oracle, acc_dtype, g_dtype):
     from flextrain_amd import _C
     lib = _C.lib()
+
+    def host(t):  # numpy view the checker takes: fp32 as it is, 16-bit types as bit patterns
+        c = t.detach().cpu().contiguous()
+        return c.numpy().copy() if c.dtype == torch.float32 else c.view(torch.int16).numpy().view(np.uint16).copy()
     stream = _C.current_stream_ptr(cuda)
     code = _C.dtype_code
     # the second call is smaller and starts at an odd element: edge elements on both sides
@@ -43,6 +51,9 @@ def test_static_scratch_entry_point_equals_the_workspace_one(cuda, acc_dtype, g_
         acc, g = _inputs(cuda, n + off, acc_dtype, g_dtype, seed=40 + k, bad=[b + off for b in bad])
         acc2, g2 = acc.clone(), g.clone()
         a, b, a2, b2 = acc[off:], g[off:], acc2[off:], g2[off:]
+        acc_host, g_host = host(a), host(b)
+        oracle.grad_accumulate(acc_host, code(acc_dtype), g_host, code(g_dtype), scale=0.25, zero_g=True)
+        bad_host, sumsq_host = oracle.grad_stats(acc_host, code(acc_dtype), pre_mult=1.0 / 64)
         want, got = _record(cuda), _record(cuda)
         ws_bytes = int(lib.ft_grad_accumulate_workspace_bytes(n))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=cuda)
@@ -61,6 +72,10 @@ def test_static_scratch_entry_point_equals_the_workspace_one(cuda, acc_dtype, g_
         hw, hg = want.cpu(), got.cpu()
         assert hw.view(torch.int64).tolist() == hg.view(torch.int64).tolist(), f"call {k}: statistics differ: {hw} / {hg}"
         assert int(hg[0:1].view(torch.int64).item()) == len(bad) and float(hg[1]) > 0.0
+        # against the CPU checker: the accumulator bit for bit, the statistics of the new accumulator
+        assert np.array_equal(host(a2), acc_host), f"call {k}: accumulator differs from the checker's"
+        assert int(hg[0:1].view(torch.int64).item()) == bad_host
+        assert abs(float(hg[1]) - sumsq_host) <= 1e-9 * sumsq_host, (float(hg[1]), sumsq_host)
     # adding to an existing record, and no statistics at all (no scratch used)
     acc, g = _inputs(cuda, 100_000, acc_dtype, g_dtype, seed=50, bad=())
     acc2, g2 = acc.clone(), g.clone()
