@@ -719,18 +719,9 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
             } else {  // buffer loads with the default cache policy: a distinct instruction, so the two paths stay two
                 const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(g + tile * kTile), 0,
                                                                                    (int)(kTile * 16), kRawBufferFlags);
-#ifdef FT_STATS_KEEP_GLOBAL
-                (void)r;
-#pragma unroll
-                for (int u = 0; u < UNROLL; ++u) w[u] = *(const volatile u32x4*)(g + base + (uint64_t)u * BLOCK);
-#else
-#ifndef FT_STATS_KEEP_AUX
-#define FT_STATS_KEEP_AUX 0
-#endif
 #pragma unroll
                 for (int u = 0; u < UNROLL; ++u)
-                    w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, FT_STATS_KEEP_AUX);
-#endif
+                    w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, 0);
             }
             uint32_t marks = 0;
 #pragma unroll
