@@ -4,7 +4,8 @@ Each seed draws a schedule the other coordinator tests do not combine: number of
 micro-batches, ragged share and group boundaries (shares that start at any element offset), where
 the state lives (HBM, pinned host memory, some of each), windows of either kind, how resident units
 are cut and on which stream they run, the accumulation type, loss scaling with an inf/nan planted
-somewhere, stepping during backward or deferred to the next forward pass with or without clipping.
+somewhere, stepping during backward, split between backward and the next forward pass (alpha), or
+deferred to the next forward pass with or without clipping.
 Bars as everywhere: fp32 state within 2 ULP, the 16-bit parameters within 1 (0 is what comes out)."""
 import math
 import os
@@ -47,6 +48,8 @@ def _draw(seed):
     cfg["scaled"] = bool(rng.integers(0, 2))
     cfg["defer"] = bool(rng.integers(0, 2))
     cfg["max_grad_norm"] = 0.05 if (cfg["defer"] and rng.integers(0, 2)) else None
+    # the share of every unit's step that runs during the next forward pass (0: all during backward)
+    cfg["alpha"] = 0.0 if cfg["defer"] or rng.integers(0, 2) else float(rng.uniform(0.02, 0.98))
     cfg["iterations"] = 3
     # (iteration, unit, micro-batch, element) of a planted inf/nan; checked only where gradients are scaled
     cfg["planted"] = (int(rng.integers(1, 4)), int(rng.integers(0, cfg["num_units"])), int(rng.integers(0, cfg["micro_batches"])),
@@ -81,7 +84,7 @@ def test_random_schedule(cuda, oracle, seed):
     coord.initialize(opt, flat, mbs, offload=cfg["offload"], device=cuda, resident_units=cfg["resident_units"],
                      unit_windows=cfg["unit_windows"], window_write_through=cfg["window_write_through"],
                      resident_shares=cfg["resident_shares"], step_stream=cfg["step_stream"], gradacc_dtype=cfg["gradacc"],
-                     loss_scaler=scaler, max_grad_norm=cfg["max_grad_norm"], defer_to_forward=cfg["defer"])
+                     loss_scaler=scaler, max_grad_norm=cfg["max_grad_norm"], defer_to_forward=cfg["defer"], alpha=cfg["alpha"])
     segments = [(bounds[k], bounds[k + 1] if k + 1 < len(bounds) - 1 else n, groups[k]) for k in range(len(groups))]
     state = [(to_np(f.float()).copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)) for f in flat]
     expected_half = [half_bits(f).copy() for f in flat]
@@ -118,11 +121,11 @@ def test_random_schedule(cuda, oracle, seed):
 
     applied, overflows = 0, []
     for iteration in range(1, cfg["iterations"] + 1):
-        if cfg["defer"]:
+        if cfg["defer"] or cfg["alpha"] > 0:
             forward_pass()
             coord.synchronize()
             check(f"before iteration {iteration}")
-        else:
+        if not cfg["defer"]:
             opt.update_states()
         scale = coord.loss_scale
         accumulated, bad_units, sumsq = {}, set(), 0.0
@@ -168,12 +171,15 @@ def test_random_schedule(cuda, oracle, seed):
             apply(range(num_units), applied, grad_mult, accumulated)
         else:
             first_bad = max(bad_units) if bad_units else -1  # that unit and every unit stepped after it are skipped
+            if bad_units and coord._defer:  # alpha rounded up to the whole slice: nothing is stepped before the global decision
+                first_bad = num_units - 1
             if scaler is not None:
                 assert coord.last_skipped_units == list(range(first_bad + 1)), cfg
             apply([u for u in range(num_units) if u > first_bad], iteration,
                   float(np.float32(1.0 / scale)) if scaler is not None else 1.0, accumulated)
-            check(f"after iteration {iteration}")
-    if cfg["defer"]:
+            if cfg["alpha"] == 0:
+                check(f"after iteration {iteration}")
+    if cfg["defer"] or cfg["alpha"] > 0:
         forward_pass()
         coord.synchronize()
         check("final")
