@@ -54,6 +54,7 @@ struct StreamState {
     void* ptr = nullptr;  // library-owned scratch, grown on demand
     size_t bytes = 0;
     int ticket_slot = -1; // index into the device's ticket pool, -1: none assigned (yet, or pool exhausted)
+    uint32_t tag = 0;     // tag of the last one-launch pass enqueued here (16 bits, never 0)
 };
 std::map<std::pair<int, hipStream_t>, StreamState> g_stream_state;
 constexpr int kTicketSlots = 1024;
@@ -476,9 +477,10 @@ std::unordered_map<int, uint32_t*> g_ticket_pool_ptr;  // device -> that device'
 // The ticket counter of (current device, stream), or nullptr when the pass has to take two launches:
 // a stream under graph capture (the recorded kernel would be replayed on whatever stream the graph is
 // launched on, beside eager passes that own this counter), or no counter left.
-int stream_ticket(hipStream_t stream, uint32_t** out)
+int stream_ticket(hipStream_t stream, uint32_t** out, uint32_t* tag)
 {
     *out = nullptr;
+    *tag = 0;
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
         (void)hipGetLastError();
@@ -505,6 +507,8 @@ int stream_ticket(hipStream_t stream, uint32_t** out)
         free_slots.pop_back();
     }
     *out = pool->second + static_cast<size_t>(st.ticket_slot) * kTicketStride;
+    st.tag = st.tag % 0xffffu + 1;  // 1 ... 65535, a new one for every pass on this stream
+    *tag = st.tag;
     return FT_OK;
 }
 
@@ -842,6 +846,7 @@ int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* 
     fin.max_norm = dec.max_norm;
     fin.ctl = dec.ctl;
     fin.ticket = nullptr;
+    fin.tag = 0;
     int blocks = 0;
     if (nvec > 0) {
         constexpr size_t kTile = static_cast<size_t>(FT_STATS_BLOCK) * FT_STATS_UNROLL;
@@ -853,7 +858,7 @@ int grad_stats_impl(const void* g, int g_dtype, size_t n, float pre_mult, void* 
         // One launch where the stream has a ticket counter of its own: the block that delivers the
         // last partial also takes the final sum (and the decision).
         if (g_stats_one_launch.load()) {
-            int trc = stream_ticket(stream, &fin.ticket);
+            int trc = stream_ticket(stream, &fin.ticket, &fin.tag);
             if (trc != FT_OK) return trc;
         }
         const ftk::u32x4* gv = reinterpret_cast<const ftk::u32x4*>(static_cast<const char*>(g) + head * esz);

@@ -563,21 +563,45 @@ __device__ __forceinline__ void block_stats_reduce(double lane_sum, uint32_t bad
 // statistics pass went from 66 to 85 us). The partial is therefore stored and loaded with
 // device-scope atomic accesses (relaxed), which bypass the per-die caches by themselves: once such a
 // store has completed (s_waitcnt), every later device-scope access on the device sees it.
-__device__ __forceinline__ void publish_partial(StatsPartial* slot, double sum, uint64_t bad)
+// The protocol checks itself: the count travels with the pass's 16-bit tag in its upper bits and
+// is stored after the sum has arrived, and the reader takes a slot only when it carries this pass's
+// tag (re-reading a bounded number of times otherwise), so that a slot that still held an earlier
+// pass's contents could never be added up unnoticed. A slot that never shows the tag -- which the
+// coherence of device-scope accesses rules out -- is reported as kPartialLost non-finite elements:
+// the step is skipped and the iteration flagged, not silently wrong.
+constexpr int kPartialTagShift = 48;                      // counts stay below 2^48 elements
+constexpr uint64_t kPartialCountMask = (1ull << kPartialTagShift) - 1;
+constexpr uint64_t kPartialLost = 1ull << 47;
+constexpr int kPartialRetries = 1 << 16;
+
+__device__ __forceinline__ void publish_partial(StatsPartial* slot, double sum, uint64_t bad, uint32_t tag)
 {
     __hip_atomic_store(reinterpret_cast<uint64_t*>(&slot->sumsq), __builtin_bit_cast(uint64_t, sum), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(&slot->nonfinite, bad, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both stores have arrived before anything below is issued
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the sum has arrived before its tagged count is issued
+    __hip_atomic_store(&slot->nonfinite, (bad & kPartialCountMask) | ((uint64_t)tag << kPartialTagShift), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // ... and that before the ticket is drawn
 }
 template <bool COHERENT>
-__device__ __forceinline__ StatsPartial read_partial(const StatsPartial* slot)
+__device__ __forceinline__ StatsPartial read_partial(const StatsPartial* slot, uint32_t tag)
 {
     if constexpr (!COHERENT) return *slot;  // written by an earlier launch
     StatsPartial r;
+    uint64_t word = 0;
+    int tries = 0;
+    do {
+        word = __hip_atomic_load(&slot->nonfinite, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } while ((uint32_t)(word >> kPartialTagShift) != tag && ++tries < kPartialRetries);
+    if ((uint32_t)(word >> kPartialTagShift) != tag) {
+        r.sumsq = 0.0;
+        r.nonfinite = kPartialLost;
+        return r;
+    }
+    asm volatile("" ::: "memory");  // the sum is loaded after the tagged count has been seen
     r.sumsq = __builtin_bit_cast(double, __hip_atomic_load(reinterpret_cast<const uint64_t*>(&slot->sumsq), __ATOMIC_RELAXED,
                                                            __HIP_MEMORY_SCOPE_AGENT));
-    r.nonfinite = __hip_atomic_load(&slot->nonfinite, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    r.nonfinite = word & kPartialCountMask;
     return r;
 }
 
@@ -629,6 +653,7 @@ struct StatsFinalArgs {
     float max_norm;
     ft_step_control_t* ctl;
     uint32_t* ticket;     // one-launch mode: counts the blocks that have delivered their partial; nullptr: two launches
+    uint32_t tag;         // one-launch mode: 16-bit tag of this pass (differs from the previous pass on the same scratch)
 };
 
 // End of a statistics pass, run by the first 256 threads of ONE block (all threads of the block must
@@ -644,7 +669,7 @@ __device__ __forceinline__ void stats_final_block(const StatsPartial* partials, 
         double s = 0.0;
         uint64_t b = 0;
         for (int i = threadIdx.x; i < nparts; i += 256) {
-            const StatsPartial part = read_partial<COHERENT>(partials + i);
+            const StatsPartial part = read_partial<COHERENT>(partials + i, f.tag);
             s += part.sumsq;
             b += part.nonfinite;
         }
@@ -756,7 +781,7 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
     // separate launch would, and leaves the ticket counter at zero for the next pass on this stream.
     __shared__ uint32_t s_last;
     if (threadIdx.x == 0) {
-        publish_partial(partials + blockIdx.x, total, total_bad);
+        publish_partial(partials + blockIdx.x, total, total_bad, fin.tag);
         s_last = __hip_atomic_fetch_add(fin.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1 ? 1u : 0u;
     }
     __syncthreads();

@@ -329,6 +329,48 @@ void accumulate_without_allocating(hipStream_t stream)
     HIP_OK(hipFree(dacc)); HIP_OK(hipFree(dg)); HIP_OK(hipFree(rec));
 }
 
+void launch_plan_and_stream_state(hipStream_t stream)
+{
+    // how work is cut into launches: plain arithmetic behind the ABI
+    uint64_t first[8], count[8];
+    check(ft_launch_pieces(10, 4, first, count, 8) == 3 && first[2] == 8 && count[2] == 2 && count[0] == 4,
+          "launch plan: 10 workgroups under a limit of 4 are pieces of 4, 4 and 2");
+    check(ft_launch_pieces((1ull << 26), 0, first, count, 8) == 2 && count[0] == (0xffffffffull / 64) && count[1] == 1,
+          "launch plan: the default limit is (2^32 - 1) / 64 workgroups");
+    const uint64_t wgs[5] = {3, 3, 3, 9, 1};
+    int batch_of[5];
+    check(ft_segment_batches(wgs, 5, 9, batch_of) == 3 && batch_of[2] == 0 && batch_of[3] == 1 && batch_of[4] == 2,
+          "segment batches: a launch of at most 9 workgroups");
+    check(ft_set_launch_limit(0xffffffffull) == FT_EINVAL && ft_set_launch_limit(0) == FT_OK, "launch limit: above the runtime's is refused");
+    // a statistics pass as one launch and as two give the same record; the stream's state can be given back
+    const size_t n = 1'000'003;
+    std::vector<uint16_t> g(n);
+    for (size_t i = 0; i < n; ++i) g[i] = static_cast<uint16_t>(0x3c00 + (i * 2654435761u >> 22));  // fp16 values in [1, 2)
+    uint16_t* dg = nullptr;
+    unsigned char* rec = nullptr;
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&dg), n * 2));
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&rec), 64));
+    HIP_OK(hipMemcpy(dg, g.data(), n * 2, hipMemcpyHostToDevice));
+    unsigned char one[32], two[32];
+    FT_OK_OR_DIE(ft_grad_decide(dg, FT_F16, n, 0.5f, rec, 0, 0.5f, 1.0f, rec + 16, nullptr, 0, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(one, rec, 32, hipMemcpyDeviceToHost));
+    FT_OK_OR_DIE(ft_set_stats_launches(2));
+    FT_OK_OR_DIE(ft_grad_decide(dg, FT_F16, n, 0.5f, rec + 32, 0, 0.5f, 1.0f, rec + 48, nullptr, 0, stream));
+    FT_OK_OR_DIE(ft_set_stats_launches(1));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(two, rec + 32, 32, hipMemcpyDeviceToHost));
+    check(!std::memcmp(one, two, 32), "statistics pass: one launch and two launches give the same 32 bytes");
+    check(ft_set_stats_launches(3) == FT_EINVAL, "statistics pass: 1 or 2 launches");
+    FT_OK_OR_DIE(ft_release_stream_scratch(stream));
+    FT_OK_OR_DIE(ft_grad_decide(dg, FT_F16, n, 0.5f, rec + 32, 0, 0.5f, 1.0f, rec + 48, nullptr, 0, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(hipMemcpy(two, rec + 32, 32, hipMemcpyDeviceToHost));
+    check(!std::memcmp(one, two, 32), "statistics pass: the same after the stream's scratch was released");
+    FT_OK_OR_DIE(ft_release_stream_scratch(stream));
+    HIP_OK(hipFree(dg)); HIP_OK(hipFree(rec));
+}
+
 void link_probe()
 {
     ft_link_probe_t r;
@@ -426,6 +468,7 @@ int main()
     accumulate_pass(stream);
     many_segments_one_launch(stream);
     accumulate_without_allocating(stream);
+    launch_plan_and_stream_state(stream);
     offloaded_step(stream);
     link_probe();
     synthetic_inputs(stream);
