@@ -88,6 +88,7 @@ EXPORTS = {
     "ft_set_launch_limit": (c_int, [c_uint64]),
     "ft_launch_pieces": (c_int, [c_uint64, c_uint64, POINTER(c_uint64), POINTER(c_uint64), c_int]),
     "ft_segment_batches": (c_int, [POINTER(c_uint64), c_int, c_uint64, POINTER(c_int)]),
+    "ft_relaxed_tile_start": (c_int, [POINTER(c_uint64), POINTER(c_uint32), POINTER(c_uint32), c_int, POINTER(c_uint32)]),
     "ft_release_stream_scratch": (c_int, [c_void_p]),
 }
 

@@ -245,12 +245,20 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
     };
 
     if (!vec_ok) {
-        // Arrays whose alignments disagree: whole tiles behind p's own head still go through a tile
-        // kernel (one that assumes element alignment only), the rest element by element.
-        const size_t head4 = ((16 - (reinterpret_cast<uintptr_t>(p) & 15)) & 15) / 4;
-        const size_t rhead = head4 < n ? head4 : n;
+        // Arrays whose alignments disagree: whole tiles still go through a tile kernel (one that
+        // assumes element alignment only), the rest element by element. The tiles start where most
+        // of the traffic is on whole cache lines (written bytes counted twice).
+        const fth::ArrayPlacement place[8] = {
+            {reinterpret_cast<uintptr_t>(out.p), 4, 8}, {reinterpret_cast<uintptr_t>(out.m), 4, 8},
+            {reinterpret_cast<uintptr_t>(out.v), 4, 8}, {reinterpret_cast<uintptr_t>(h), 2, h ? 4u : 0u},
+            {reinterpret_cast<uintptr_t>(p), 4, 4},     {reinterpret_cast<uintptr_t>(m), 4, 4},
+            {reinterpret_cast<uintptr_t>(v), 4, 4},     {reinterpret_cast<uintptr_t>(g), static_cast<uint32_t>(gsz), static_cast<uint32_t>(gsz)}};
+        uint32_t on_lines = 0;
+        const size_t head_r = fth::plan_relaxed_head(place, 8, &on_lines);
+        const size_t rhead = head_r < n ? head_r : n;
         const size_t rtiles = (n - rhead) / 4 / ftk::kWave;
         if (rtiles == 0) return scalar_part(0, n);
+        if (!h) on_lines &= ~8u;
         ftk::AdamArgs a;
         a.p = p + rhead;
         a.g = gb + rhead * gsz;
@@ -269,10 +277,10 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         for (uint64_t piece = 0; plan_launch_piece(rtiles, launch_limit(), piece, &tile0, &blocks); ++piece) {
             if (ctl)
                 hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, true>), dim3(static_cast<unsigned>(blocks)), dim3(ftk::kWave),
-                                   lds, stream, a, tile0);
+                                   lds, stream, a, tile0, on_lines & 15u);
             else
                 hipLaunchKernelGGL((ftk::adam_tile_relaxed_kernel<GT, HT, false>), dim3(static_cast<unsigned>(blocks)), dim3(ftk::kWave),
-                                   lds, stream, a, tile0);
+                                   lds, stream, a, tile0, on_lines & 15u);
             FT_HIP(hipGetLastError());
         }
         const size_t rbody = rtiles * ftk::kWave * 4;
@@ -1074,6 +1082,17 @@ int ft_segment_batches(const uint64_t* workgroups, int n_segs, uint64_t limit, i
     if (n_segs < 0 || (n_segs > 0 && (!workgroups || !batch_of))) return fth::fail(FT_EINVAL, "bad arguments");
     if (limit == 0) limit = multi_launch_limit();
     return fth::plan_segment_batches(workgroups, n_segs, ftk::kMultiMaxSegments, limit, batch_of);
+}
+
+int ft_relaxed_tile_start(const uint64_t* addresses, const uint32_t* elem_bytes, const uint32_t* weights, int count, uint32_t* on_lines)
+{
+    if (count < 1 || count > 32 || !addresses || !elem_bytes || !weights || !on_lines) return fth::fail(FT_EINVAL, "bad arguments");
+    fth::ArrayPlacement place[32];
+    for (int k = 0; k < count; ++k) {
+        if (elem_bytes[k] != 2 && elem_bytes[k] != 4) return fth::fail(FT_EINVAL, "array %d: element size %u", k, elem_bytes[k]);
+        place[k] = {addresses[k], elem_bytes[k], weights[k]};
+    }
+    return static_cast<int>(fth::plan_relaxed_head(place, count, on_lines));
 }
 
 int ft_set_stats_launches(int launches)

@@ -52,4 +52,46 @@ inline int plan_segment_batches(const uint64_t* wgs, int n, int max_segs, uint64
     return n > 0 ? batch + 1 : 0;
 }
 
+// Where the tiles of a step start when its arrays do not reach their vector alignment together.
+// One array per entry: its address, its element size (2 or 4 bytes) and a weight (bytes moved per
+// element, written bytes counted twice: a store that covers part of a cache line costs more than a
+// load that does). Tiles are 256 elements, so a choice of `head` elements in front of the first
+// tile fixes, for every array, whether its tiles start on 128-byte lines (whole-line traffic) and
+// whether its 4-element units are aligned as vectors. Returns the head below 64 (the period of a
+// 2-byte array's line phase) with the largest weighted score, the smallest such on a tie, and the
+// set of arrays whose tiles then start on lines (bit k: array k).
+struct ArrayPlacement {
+    uint64_t address;
+    uint32_t elem_bytes;
+    uint32_t weight;
+};
+constexpr uint32_t kLineBytes = 128;
+constexpr uint32_t kRelaxedHeadPeriod = 64;
+
+inline uint32_t plan_relaxed_head(const ArrayPlacement* arrays, int count, uint32_t* on_lines)
+{
+    uint32_t best_head = 0, best_mask = 0;
+    uint64_t best_score = 0;
+    for (uint32_t head = 0; head < kRelaxedHeadPeriod; ++head) {
+        uint64_t score = 0;
+        uint32_t mask = 0;
+        for (int k = 0; k < count; ++k) {
+            const uint64_t at = arrays[k].address + static_cast<uint64_t>(head) * arrays[k].elem_bytes;
+            if (at % kLineBytes == 0) {
+                score += 4ull * arrays[k].weight;
+                mask |= 1u << k;
+            } else if (at % (4ull * arrays[k].elem_bytes) == 0) {
+                score += arrays[k].weight;
+            }
+        }
+        if (head == 0 || score > best_score) {
+            best_head = head;
+            best_score = score;
+            best_mask = mask;
+        }
+    }
+    *on_lines = best_mask;
+    return best_head;
+}
+
 }  // namespace fth

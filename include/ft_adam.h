@@ -87,9 +87,11 @@ int ft_adam_destroy(int id);
  * front of the first 1 KiB boundary of p and behind the last whole 256-element tile separately
  * (same launch for an in-place update) so that every tile covers whole cache lines. Arrays whose
  * alignments disagree (a 16-bit copy cut at an odd element, a state array one element off) are still
- * stepped tile by tile, through accesses that assume element alignment only: the same results, at
- * 77-82 % of the memory bandwidth instead of 85 % (measured with one array of a 202 M-element update
- * one element off the others).
+ * stepped tile by tile, through accesses that assume element alignment only; the tiles then start
+ * where most of the traffic falls on whole cache lines (written bytes counted twice), see
+ * ft_relaxed_tile_start. The same results, at 80-84 % of the memory bandwidth instead of 84-86 %
+ * (measured with one array of a 202 M-element update one element off the others; 70-77 % with
+ * every array at another offset).
  */
 int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, float eps,
                  float weight_decay, int bias_correction, float grad_mult, void* p, const void* g,
@@ -358,10 +360,18 @@ int ft_set_cache_tuning(size_t stats_keep_bytes);
  * ordinary sizes; results never depend on it. ft_launch_pieces reports how `workgroups` workgroups
  * are cut under `limit` (0 = the current one): first[k], count[k] for piece k, at most `capacity`
  * of them; returns the number of pieces. ft_segment_batches reports which launch each of n_segs
- * segments (workgroups[i] workgroups each) of a many-segment call falls into. Neither touches a GPU. */
+ * segments (workgroups[i] workgroups each) of a many-segment call falls into.
+ * ft_relaxed_tile_start reports where ft_adam_step starts its 256-element tiles when the arrays of
+ * a step do not reach their vector alignment together: given each array's address, element size (2
+ * or 4) and weight (bytes moved per element, written bytes twice), the number of elements (below 64)
+ * left in front of the first tile so that as much of the traffic as possible is on whole 128-byte
+ * lines, and in *on_lines the arrays (bit k: array k) whose tiles then start on lines. None of the
+ * three touches a GPU. */
 int ft_set_launch_limit(uint64_t max_workgroups);
 int ft_launch_pieces(uint64_t workgroups, uint64_t limit, uint64_t* first, uint64_t* count, int capacity);
 int ft_segment_batches(const uint64_t* workgroups, int n_segs, uint64_t limit, int* batch_of);
+int ft_relaxed_tile_start(const uint64_t* addresses, const uint32_t* elem_bytes, const uint32_t* weights, int count,
+                          uint32_t* on_lines);
 /* launches: 1 (default) = the statistics pass as one kernel launch, 2 = the partial sums and the
  * final sum as two launches (what a stream under graph capture always gets). Same results. */
 int ft_set_stats_launches(int launches);

@@ -89,3 +89,64 @@ def test_segment_batches_respect_both_limits(lib):
     # and what the runtime accepts
     n, batch_of = _batches(lib, [MAX_WORKGROUPS - 1, 1, 1], 0)
     assert batch_of == [0, 0, 1]
+
+
+# ---- where relaxed-alignment tiles start -----------------------------------------------------------
+def _tile_start(lib, arrays):
+    """arrays: [(address, element bytes, weight)] -> (head, set of array indices whose tiles start on lines)"""
+    n = len(arrays)
+    addr = (ctypes.c_uint64 * n)(*[a for a, _, _ in arrays])
+    width = (ctypes.c_uint32 * n)(*[w for _, w, _ in arrays])
+    weight = (ctypes.c_uint32 * n)(*[w for _, _, w in arrays])
+    mask = ctypes.c_uint32(0xffffffff)
+    head = lib.ft_relaxed_tile_start(addr, width, weight, n, ctypes.byref(mask))
+    assert 0 <= head < 64, head
+    on = {k for k in range(n) if mask.value >> k & 1}
+    assert mask.value >> n == 0
+    for k, (a, w, _) in enumerate(arrays):  # the mask says exactly which arrays sit on 128-byte lines behind the head
+        assert ((a + head * w) % 128 == 0) == (k in on), (k, head)
+    return head, on
+
+
+BASE = 0x7f00_0000_0000
+
+
+def test_arrays_with_a_common_phase_all_start_on_lines(lib):
+    for cut in (0, 1, 5, 31, 33, 63, 64, 100, 255):
+        arrays = [(BASE + (k << 30) + cut * w, w, 4) for k, w in enumerate((4, 4, 4, 2, 2))]
+        head, on = _tile_start(lib, arrays)
+        assert on == {0, 1, 2, 3, 4} and head == (-cut) % 64, (cut, head)
+
+
+@pytest.mark.parametrize("odd", range(5))
+@pytest.mark.parametrize("shift", [1, 2, 3, 7, 40])
+def test_one_array_off_leaves_the_others_on_lines(lib, odd, shift):
+    widths = (4, 4, 4, 2, 2)
+    arrays = [(BASE + (k << 30) + (shift * w if k == odd else 0), w, 8 if k < 3 else 2) for k, w in enumerate(widths)]
+    head, on = _tile_start(lib, arrays)
+    assert head == 0 and on == set(range(5)) - {odd}
+
+
+def test_the_heavier_side_wins_and_ties_take_the_smaller_head(lib):
+    # written state (weight 8 each) three elements in, gradient and copy (weight 2 each) at the start
+    arrays = [(BASE + 12, 4, 8), (BASE + (1 << 30) + 12, 4, 8), (BASE + (2 << 30), 2, 2), (BASE + (3 << 30), 2, 2)]
+    head, on = _tile_start(lib, arrays)
+    assert head == 29 and on == {0, 1}
+    # equal weights on both sides: both heads score the same, the smaller one is taken
+    arrays = [(BASE + 12, 4, 8), (BASE + (1 << 30), 4, 8)]
+    head, on = _tile_start(lib, arrays)
+    assert head == 0 and on == {1}
+    # nothing can be put on a line (dword-aligned fp32 arrays at different phases of 16 bytes):
+    # the head that at least makes the heavier one's 4-element units whole vectors
+    arrays = [(BASE + 4, 4, 8), (BASE + (1 << 30) + 8, 4, 2)]
+    head, on = _tile_start(lib, arrays)
+    assert on == {0} and head == 31  # 31 elements later the first array IS on a line
+
+
+def test_tile_start_refuses_bad_arguments(lib):
+    mask = ctypes.c_uint32()
+    a, w, g = (ctypes.c_uint64 * 1)(BASE), (ctypes.c_uint32 * 1)(3), (ctypes.c_uint32 * 1)(1)
+    assert lib.ft_relaxed_tile_start(a, w, g, 1, ctypes.byref(mask)) < 0
+    w[0] = 4
+    assert lib.ft_relaxed_tile_start(a, w, g, 0, ctypes.byref(mask)) < 0
+    assert lib.ft_relaxed_tile_start(a, w, g, 1, ctypes.byref(mask)) == 0 and mask.value == 1
