@@ -36,7 +36,7 @@
 #define FT_STATS_UNROLL 4
 #endif
 #ifndef FT_STATS_BLOCKS_PER_CU
-#define FT_STATS_BLOCKS_PER_CU 3
+#define FT_STATS_BLOCKS_PER_CU 2
 #endif
 
 namespace {

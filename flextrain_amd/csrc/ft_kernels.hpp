@@ -15,6 +15,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #include "ft_adam.h"
 #include "ft_types.hpp"
@@ -490,6 +491,19 @@ __device__ __forceinline__ double wave_sum_f64(double x)
     return (readlane_f64(x, 0) + readlane_f64(x, 16)) + (readlane_f64(x, 32) + readlane_f64(x, 48));
 }
 
+__device__ __forceinline__ uint64_t wave_sum_u64(uint64_t x)
+{
+    auto permuted = [](uint64_t v, auto ctrl) {
+        return __builtin_bit_cast(uint64_t, dpp_f64<decltype(ctrl)::value>(__builtin_bit_cast(double, v)));
+    };
+    x += permuted(x, std::integral_constant<int, 0xB1>{});
+    x += permuted(x, std::integral_constant<int, 0x4E>{});
+    x += permuted(x, std::integral_constant<int, 0x141>{});
+    x += permuted(x, std::integral_constant<int, 0x140>{});
+    auto lane = [&](const int l) { return __builtin_bit_cast(uint64_t, readlane_f64(__builtin_bit_cast(double, x), l)); };
+    return lane(0) + lane(16) + lane(32) + lane(48);
+}
+
 // x*x added to acc in fp64. The square of an fp32 value is exact in fp64 (24-bit significand), so
 // the only rounding is the addition's, and no finite fp32 value can make the sum overflow or vanish:
 // 3.4e38 squared is 1.2e77, 1.4e-45 squared 2e-90, both far inside the fp64 range.
@@ -567,24 +581,26 @@ __device__ __forceinline__ void stats_accumulate_finite(u32x4 w, float pre_mult,
 template <int BLOCK>
 __device__ __forceinline__ void block_stats_reduce(double lane_sum, uint32_t bad, double& total, uint64_t& total_bad)
 {
-    __shared__ double s_sum[BLOCK];
+    __shared__ double s_sum[BLOCK / kWave];
     __shared__ uint32_t s_bad[BLOCK / kWave];
+    const double ts = wave_sum_f64(lane_sum);
     const uint32_t tb = wave_sum_u32(bad);
-    s_sum[threadIdx.x] = lane_sum;
-    if ((threadIdx.x & (kWave - 1)) == 0) s_bad[threadIdx.x / kWave] = tb;
-    __syncthreads();
-#pragma unroll
-    for (int w = BLOCK / 2; w > 0; w >>= 1) {
-        if ((int)threadIdx.x < w) s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
-        __syncthreads();
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        s_sum[threadIdx.x / kWave] = ts;
+        s_bad[threadIdx.x / kWave] = tb;
     }
+    __syncthreads();
     total = 0.0;
     total_bad = 0;
     if (threadIdx.x == 0) {
-        uint64_t b = 0;
+        double t = s_sum[0];
+        uint64_t b = s_bad[0];
 #pragma unroll
-        for (int k = 0; k < BLOCK / kWave; ++k) b += s_bad[k];
-        total = s_sum[0];
+        for (int k = 1; k < BLOCK / kWave; ++k) {
+            t += s_sum[k];
+            b += s_bad[k];
+        }
+        total = t;
         total_bad = b;
     }
 }
@@ -595,12 +611,13 @@ __device__ __forceinline__ void block_stats_reduce(double lane_sum, uint32_t bad
 // statistics pass went from 66 to 85 us). The partial is therefore stored and loaded with
 // device-scope atomic accesses (relaxed), which bypass the per-die caches by themselves: once such a
 // store has completed (s_waitcnt), every later device-scope access on the device sees it.
-// The protocol checks itself: the count travels with the pass's 16-bit tag in its upper bits and
-// is stored after the sum has arrived, and the reader takes a slot only when it carries this pass's
-// tag (re-reading a bounded number of times otherwise), so that a slot that still held an earlier
-// pass's contents could never be added up unnoticed. A slot that never shows the tag -- which the
-// coherence of device-scope accesses rules out -- is reported as kPartialLost non-finite elements:
-// the step is skipped and the iteration flagged, not silently wrong.
+// A block draws its ticket only after both words of its partial have completed, so the block that
+// draws the last ticket finds every partial whole. The protocol checks itself all the same: the
+// count travels with the pass's 16-bit tag in its upper bits, and the reader takes a slot only when
+// it carries this pass's tag (re-reading a bounded number of times otherwise), so that a slot that
+// still held an earlier pass's contents could never be added up unnoticed. A slot that never shows
+// the tag -- which the coherence of device-scope accesses rules out -- is reported as kPartialLost
+// non-finite elements: the step is skipped and the iteration flagged, not silently wrong.
 constexpr int kPartialTagShift = 48;                      // counts stay below 2^48 elements
 constexpr uint64_t kPartialCountMask = (1ull << kPartialTagShift) - 1;
 constexpr uint64_t kPartialLost = 1ull << 47;
@@ -610,15 +627,13 @@ __device__ __forceinline__ void publish_partial(StatsPartial* slot, double sum, 
 {
     __hip_atomic_store(reinterpret_cast<uint64_t*>(&slot->sumsq), __builtin_bit_cast(uint64_t, sum), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the sum has arrived before its tagged count is issued
     __hip_atomic_store(&slot->nonfinite, (bad & kPartialCountMask) | ((uint64_t)tag << kPartialTagShift), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // ... and that before the ticket is drawn
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // both have arrived before the ticket is drawn
 }
-template <bool COHERENT>
-__device__ __forceinline__ StatsPartial read_partial(const StatsPartial* slot, uint32_t tag)
+// One slot, patiently: for a slot that did not show this pass's tag at the first look.
+__device__ __forceinline__ StatsPartial reread_partial(const StatsPartial* slot, uint32_t tag)
 {
-    if constexpr (!COHERENT) return *slot;  // written by an earlier launch
     StatsPartial r;
     uint64_t word = 0;
     int tries = 0;
@@ -635,6 +650,50 @@ __device__ __forceinline__ StatsPartial read_partial(const StatsPartial* slot, u
                                                            __HIP_MEMORY_SCOPE_AGENT));
     r.nonfinite = word & kPartialCountMask;
     return r;
+}
+// Thread t of 256 adds up partials t, t + 256, ... in that order. The loads of four slots are issued
+// together and looked at afterwards: the block that runs this has just waited for the last partial,
+// and a round trip to device-coherent memory per slot and word (four in a row for 512 partials) would
+// be most of what the final sum costs.
+template <bool COHERENT>
+__device__ __forceinline__ void sum_partials(const StatsPartial* partials, int nparts, uint32_t tag, double& s, uint64_t& b)
+{
+    constexpr int kBatch = 4;
+    s = 0.0;
+    b = 0;
+    for (int first = threadIdx.x; first < nparts; first += 256 * kBatch) {
+        uint64_t word[kBatch], sum[kBatch];
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k) {
+            const int i = first + k * 256;
+            word[k] = sum[k] = 0;
+            if (i < nparts) {
+                if constexpr (COHERENT) {
+                    word[k] = __hip_atomic_load(&partials[i].nonfinite, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    sum[k] = __hip_atomic_load(reinterpret_cast<const uint64_t*>(&partials[i].sumsq), __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                } else {  // written by an earlier launch
+                    word[k] = partials[i].nonfinite;
+                    sum[k] = __builtin_bit_cast(uint64_t, partials[i].sumsq);
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; ++k) {
+            const int i = first + k * 256;
+            if (i < nparts) {
+                StatsPartial part;
+                part.sumsq = __builtin_bit_cast(double, sum[k]);
+                part.nonfinite = word[k];
+                if constexpr (COHERENT) {
+                    part.nonfinite = word[k] & kPartialCountMask;
+                    if ((uint32_t)(word[k] >> kPartialTagShift) != tag) part = reread_partial(partials + i, tag);
+                }
+                s += part.sumsq;
+                b += part.nonfinite;
+            }
+        }
+    }
 }
 
 // The per-step decision from a statistics record (one thread):
@@ -695,30 +754,23 @@ struct StatsFinalArgs {
 template <int GT, bool COHERENT>
 __device__ __forceinline__ void stats_final_block(const StatsPartial* partials, int nparts, float pre_mult, const StatsFinalArgs& f)
 {
-    __shared__ double s_fsum[256];
-    __shared__ uint64_t s_fbad[256];
+    __shared__ double s_fsum[4];
+    __shared__ uint64_t s_fbad[4];
     if (threadIdx.x < 256) {
-        double s = 0.0;
-        uint64_t b = 0;
-        for (int i = threadIdx.x; i < nparts; i += 256) {
-            const StatsPartial part = read_partial<COHERENT>(partials + i, f.tag);
-            s += part.sumsq;
-            b += part.nonfinite;
+        double s;
+        uint64_t b;
+        sum_partials<COHERENT>(partials, nparts, f.tag, s, b);
+        s = wave_sum_f64(s);
+        b = wave_sum_u64(b);
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            s_fsum[threadIdx.x / kWave] = s;
+            s_fbad[threadIdx.x / kWave] = b;
         }
-        s_fsum[threadIdx.x] = s;
-        s_fbad[threadIdx.x] = b;
     }
     __syncthreads();
-    for (int w = 128; w > 0; w >>= 1) {
-        if ((int)threadIdx.x < w) {
-            s_fsum[threadIdx.x] += s_fsum[threadIdx.x + w];
-            s_fbad[threadIdx.x] += s_fbad[threadIdx.x + w];
-        }
-        __syncthreads();
-    }
     if (threadIdx.x == 0) {
-        double s = s_fsum[0];
-        uint64_t b = s_fbad[0];
+        double s = (s_fsum[0] + s_fsum[1]) + (s_fsum[2] + s_fsum[3]);
+        uint64_t b = (s_fbad[0] + s_fbad[1]) + (s_fbad[2] + s_fbad[3]);
         for (uint64_t i = 0; i < f.n; ++i) {
             if (i == f.head) i = f.tail_begin;  // skip the vector body
             if (i >= f.n) break;
@@ -747,8 +799,8 @@ __device__ __forceinline__ void stats_final_block(const StatsPartial* partials, 
 // handles the elements outside [0, nvec*per_unit) in grad_stats_final_kernel.
 // Every square is formed and added in fp64 (four accumulators per lane), in the vector body as in
 // the edges, so an element contributes the same whatever part of the call it falls into, and no
-// finite gradient can overflow the sum or vanish from it. A tile's loads are first screened for
-// inf/nan as a whole; only a lane that holds one takes the per-element path that counts and masks.
+// finite gradient can overflow the sum or vanish from it. The sums are the same bits whichever of the
+// two ways below a block takes: both add an element's square to the same accumulator in the same order.
 // The gradients are read again by the update that follows the decision, so what of them still fits
 // the memory-side cache afterwards is worth keeping there: tiles from `keep_from_tile` on (the last
 // ones this pass touches) are read with ordinary loads, everything before with streaming loads that
@@ -765,37 +817,56 @@ __global__ __launch_bounds__(BLOCK) void grad_stats_kernel(const u32x4* __restri
     double acc[4] = {0.0, 0.0, 0.0, 0.0};
     uint32_t bad = 0;
     constexpr uint64_t kTile = (uint64_t)BLOCK * UNROLL;
-    const uint64_t ntiles = (nvec + kTile - 1) / kTile;
-    for (uint64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+    const uint64_t full_tiles = nvec / kTile;
+    const uint64_t stream_tiles = keep_from_tile < full_tiles ? keep_from_tile : full_tiles;
+    // The optimistic pass: whole tiles only, no branch inside a loop body (a body that first screens
+    // its loads and then chooses between two ways of adding them has to wait for all of a tile's loads
+    // before it can start on the first, and took 4-15 us more over 405 MB than one that simply adds:
+    // 62-76 against 57.5 us). Every load is added as if finite, and its inf/nan marks are collected on
+    // the side; a block that has seen a mark throws its sums away and goes over its tiles again, element
+    // by element (an overflow step is thrown away as a whole anyway, and costs this block its share of
+    // the pass a second time).
+    uint32_t marks = 0;
+    uint64_t tile = blockIdx.x;
+    for (; tile < stream_tiles; tile += gridDim.x) {
         const uint64_t base = tile * kTile + threadIdx.x;
-        if ((tile + 1) * kTile <= nvec) {
-            u32x4 w[UNROLL];
-            if (tile < keep_from_tile) {
+        u32x4 w[UNROLL];
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) w[u] = __builtin_nontemporal_load(g + base + (uint64_t)u * BLOCK);
-            } else {  // buffer loads with the default cache policy: a distinct instruction, so the two paths stay two
-                const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(g + tile * kTile), 0,
-                                                                                   (int)(kTile * 16), kRawBufferFlags);
+        for (int u = 0; u < UNROLL; ++u) w[u] = __builtin_nontemporal_load(g + base + (uint64_t)u * BLOCK);
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u)
-                    w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, 0);
-            }
-            uint32_t marks = 0;
+        for (int u = 0; u < UNROLL; ++u) {
+            marks |= nonfinite_marks<GT>(w[u]);
+            stats_accumulate_finite<GT>(w[u], pre_mult, acc);
+        }
+    }
+    for (; tile < full_tiles; tile += gridDim.x) {  // buffer loads with the default cache policy: a distinct instruction
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(g + tile * kTile), 0,
+                                                                           (int)(kTile * 16), kRawBufferFlags);
+        u32x4 w[UNROLL];
 #pragma unroll
-            for (int u = 0; u < UNROLL; ++u) marks |= nonfinite_marks<GT>(w[u]);
-            if (marks == 0) {
+        for (int u = 0; u < UNROLL; ++u)
+            w[u] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)((threadIdx.x + u * BLOCK) * 16), 0, 0);
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) stats_accumulate_finite<GT>(w[u], pre_mult, acc);
-            } else {
+        for (int u = 0; u < UNROLL; ++u) {
+            marks |= nonfinite_marks<GT>(w[u]);
+            stats_accumulate_finite<GT>(w[u], pre_mult, acc);
+        }
+    }
+    if (__syncthreads_or(marks != 0)) {  // rare: the same tiles in the same order, every element tested
+        acc[0] = acc[1] = acc[2] = acc[3] = 0.0;
+        for (tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
+            const uint64_t base = tile * kTile + threadIdx.x;
 #pragma unroll
-                for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(w[u], pre_mult, acc, bad);
-            }
-        } else {
-            for (int u = 0; u < UNROLL; ++u) {
-                const uint64_t i = base + (uint64_t)u * BLOCK;
-                if (i >= nvec) break;
-                stats_accumulate<GT>(g[i], pre_mult, acc, bad);
-            }
+            for (int u = 0; u < UNROLL; ++u) stats_accumulate<GT>(g[base + (uint64_t)u * BLOCK], pre_mult, acc, bad);
+        }
+    }
+    // the units behind the last whole tile go to the block whose turn that tile would have been
+    if (tile == full_tiles) {
+        const uint64_t base = tile * kTile + threadIdx.x;
+        for (int u = 0; u < UNROLL; ++u) {
+            const uint64_t i = base + (uint64_t)u * BLOCK;
+            if (i >= nvec) break;
+            stats_accumulate<GT>(g[i], pre_mult, acc, bad);
         }
     }
     double total;
