@@ -52,6 +52,8 @@ int cu_count();  // compute units of the current device (cached)
 
 // Dynamic LDS per 64-lane workgroup that keeps the bytes in flight per CU at the tuned level for a
 // kernel whose lanes each have `load_bytes_per_lane` bytes of loads outstanding.
-unsigned throttle_lds_bytes(unsigned load_bytes_per_lane);
+// `percent` scales the resulting number of resident wavefronts (a measured correction for a kernel
+// whose stores weigh differently).
+unsigned throttle_lds_bytes(unsigned load_bytes_per_lane, unsigned percent = 100);
 
 }  // namespace fth
