@@ -28,7 +28,7 @@ N_70B_LAYER = 2 * 8192 ** 2 + 2 * 8192 * 1024 + 3 * 8192 * 28672 + 2 * 8192  # 8
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see the summaries under
 # profiles/); None until measured for a workload.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_668_000, "cfg3": 5_666_672_000, "cfg4": 23_958_226_000, "accumulate": 2_453_896_000,
+MEASURED_TRAFFIC_BYTES = {"cfg2": 5_666_668_000, "cfg3": 5_666_667_000, "cfg4": 23_958_234_000, "accumulate": 2_453_896_000,
                           "multi": 5_666_709_000}
 # The summary each literal is copied from; it carries the line "roofline.traffic = <bytes> B"
 # (tests/test_bench_contract.py checks that the two agree).
