@@ -357,6 +357,25 @@ def bench_offload(args, torch, dev) -> int:
     return 0 if ok else 3
 
 
+def bench_ceilings() -> int:
+    """The library's kernels beside bare kernels of the same memory traffic: runs
+    flextrain_amd/ft_ceiling (a HIP program of its own, started before this process touches the
+    GPU) and prints what it measured as one JSON line."""
+    import subprocess
+
+    from flextrain_amd.build import CEILING_PATH, build_ceiling
+    if not os.path.exists(CEILING_PATH):  # nothing built in this tree yet
+        build_ceiling()
+    run = subprocess.run([CEILING_PATH], capture_output=True, text=True, timeout=300)
+    if run.returncode != 0:
+        print(run.stdout + run.stderr, file=sys.stderr)
+        return run.returncode or 1
+    cases = [json.loads(line) for line in run.stdout.splitlines() if line.startswith("{")]
+    print(json.dumps({"metric": "kernel time against a bare kernel of the same traffic, 7B-layer partition", "unit": "us",
+                      "data": "synthetic", "n_gpus": 1, "cases": cases}), flush=True)
+    return 0
+
+
 def measure_accumulate(torch, dev, steps, warmup, calibration_copy=False):
     """Gradient hand-off before the step: fp32 accumulator += bf16 micro-batch gradient over the
     7B-layer partition, clearing the source and gathering the overflow/norm statistics of the
@@ -882,7 +901,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate", "resident7b", "multi"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate", "resident7b", "multi", "ceilings"])
     ap.add_argument("--segments", type=int, default=16, help="multi: ragged contexts the partition is cut into")
     ap.add_argument("--micro-batches", type=int, default=4, help="pipeline: shares per unit")
     ap.add_argument("--windows", default="auto", choices=["auto", "off", "write_through", "copy_back"],
@@ -925,6 +944,9 @@ def main() -> int:
         print("bench.py measures the optimizer step of ONE GPU's partition; --gpus must be 1 "
               "(the path shards by giving each GPU its own slice; no multi-GPU figure exists).", file=sys.stderr)
         return 2
+
+    if args.workload == "ceilings":
+        return bench_ceilings()
 
     import torch
     if not torch.cuda.is_available():

@@ -59,5 +59,21 @@ def build_library(verbose: bool = False, extra_flags=()) -> str:
     return LIB_PATH
 
 
+CEILING_PATH = os.path.join(_PKG, "ft_ceiling")
+
+
+def build_ceiling() -> str:
+    """Compile ft_ceiling: a program that times the library's kernels (the same device code, from
+    the same header, with the same flags) beside bare kernels of the same memory traffic. Used by
+    ``bench.py --workload ceilings`` and by the relative speed floors of the GPU tests."""
+    flags = [f for f in HIPCC_FLAGS if f != "-fPIC"]
+    cmd = [hipcc(), *flags, "-I", INCLUDE, "-I", CSRC, os.path.join(CSRC, "ft_ceiling.hip"), "-o", CEILING_PATH]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on ft_ceiling.hip:\n{res.stderr}")
+    return CEILING_PATH
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_ceiling())
