@@ -222,6 +222,26 @@ int main(int argc, char** argv)
                                (uint64_t)0);
         });
         report("update, bf16 gradients and copy (adam_tile_kernel)", n * 28.0, bare, shipped);
+
+        // the same update with one array one element off the others (the relaxed-alignment tiles),
+        // against the same bare kernel on aligned arrays: what the odd array costs
+        AdamArgs b = a;
+        b.m = m + 1;  // the allocation has room behind every array
+        b.m_out = m + 1;
+        const uint32_t m_off = kRelaxedOnLinesP | kRelaxedOnLinesV | kRelaxedOnLinesH | (1u << kRelaxedCachedShift);
+        const Timing relaxed_m = time_launches([&] {
+            hipLaunchKernelGGL((adam_tile_relaxed_kernel<FT_BF16, FT_BF16, false, 1>), dim3((unsigned)tiles), dim3(kWave), lds, 0, b,
+                               (uint64_t)0, m_off);
+        });
+        report("update, m one element off (adam_tile_relaxed_kernel, that array cached)", n * 28.0, bare, relaxed_m);
+        b = a;
+        b.g = g + 1;
+        const uint32_t g_off = kRelaxedOnLinesP | kRelaxedOnLinesM | kRelaxedOnLinesV | kRelaxedOnLinesH;
+        const Timing relaxed_g = time_launches([&] {
+            hipLaunchKernelGGL((adam_tile_relaxed_kernel<FT_BF16, FT_BF16, false, 2>), dim3((unsigned)tiles), dim3(kWave), lds, 0, b,
+                               (uint64_t)0, g_off);
+        });
+        report("update, g one element off (adam_tile_relaxed_kernel, gradient cached)", n * 28.0, bare, relaxed_g);
     }
 
     // ---- accumulation (10 and 12 B/element): acc = p's array, fp32; g bf16 ---------------------------

@@ -230,21 +230,34 @@ __global__ __launch_bounds__(kWave) void adam_tile_kernel(AdamArgs a, uint64_t t
 // element, a state array one element off): the same tile shape, but every array is accessed through
 // vector types that promise only the alignment of one element, so the compiler emits whatever the
 // hardware takes at that alignment (whole 16-byte accesses at dword alignment, split ones below it).
-// Two things keep it near the aligned kernel although tiles of some arrays start inside a cache line:
-// * on_lines (bit 0 p_out, 1 m_out, 2 v_out, 3 h) names the outputs whose tiles do start on lines:
-//   those are stored like the aligned kernel's (write-through streaming stores); the others get
-//   non-temporal stores that the L2 may hold until the neighbouring tile has filled the line;
-// * workgroups go to the eight dies in turn and each die has an L2 of its own, so inside every group
-//   of 64 workgroups, workgroup r takes tile (r mod 8) * 8 + r / 8 of the group: eight consecutive
-//   tiles run on one die back to back, and seven of eight shared edge lines are completed (loads:
-//   found) in one L2 instead of going to memory twice. Workgroups behind the last whole group take
-//   their own index. Measured on the 7B-layer partition: every array at another offset 1.06 ms ->
-//   0.91 ms; longer runs cost the arrays that are aligned more than they save.
+// An array whose tiles start inside a cache line shares a line with the neighbouring tile at either
+// end; the template parameter CACHED and `flags` say how each array is treated so that this costs
+// as little as it can (what the host chooses, and why, is at its call site; all of it is measured,
+// none of it changes a result):
+// * kRelaxedOnLines bits (p_out, m_out, v_out, h): the output's tiles do start on lines and it is
+//   stored like the aligned kernel's (write-through streaming stores); the others get non-temporal
+//   stores that the L2 may hold until the neighbouring tile has filled the line;
+// * CACHED == 1: one of p, m, v (which: kRelaxedCachedShift) is read with the default cache policy,
+//   so that the second reader of a shared line finds it in a cache, instead of streaming;
+//   CACHED == 2: the gradient is. Variants of their own whose loads are always the same
+//   instructions (for the state arrays with the pointers chosen by scalar selects): a run-time
+//   choice of the load instruction per array made the compiler wait for each load before issuing the
+//   next (0.93 ms instead of 0.84), and the same global load with and without the streaming hint in
+//   two branches gets merged into one without it (hence buffer loads for the cached kind);
+// * kRelaxedCopyCached: the 16-bit copy, off the lines, is stored with the default cache policy;
+// * kRelaxedRuns: workgroups go to the eight dies in turn and each die has an L2 of its own, so
+//   inside every group of 64 workgroups, workgroup r takes tile (r mod 8) * 8 + r / 8 of the group:
+//   eight consecutive tiles run on one die back to back, and seven of eight shared edge lines are
+//   completed (loads: found) in one L2. Workgroups behind the last whole group take their own index.
 // The scalars may come from a.hyper.
 typedef float f32x4_e __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint16_t u16x4_e __attribute__((ext_vector_type(4), aligned(2)));
 constexpr uint32_t kRelaxedRun = 8;                 // consecutive tiles per die
 constexpr uint32_t kRelaxedGroup = 8 * kRelaxedRun;  // workgroups permuted among themselves
+constexpr uint32_t kRelaxedOnLinesP = 1u, kRelaxedOnLinesM = 2u, kRelaxedOnLinesV = 4u, kRelaxedOnLinesH = 8u;
+constexpr uint32_t kRelaxedCachedShift = 4;  // bits 4-5, CACHED == 1 only: 0 p, 1 m, 2 v
+constexpr uint32_t kRelaxedCopyCached = 1u << 6;
+constexpr uint32_t kRelaxedRuns = 1u << 31;
 
 __device__ __forceinline__ uint32_t relaxed_tile_of_workgroup(uint32_t b, uint32_t workgroups)
 {
@@ -253,61 +266,96 @@ __device__ __forceinline__ uint32_t relaxed_tile_of_workgroup(uint32_t b, uint32
     return (b & ~(kRelaxedGroup - 1)) + (r & 7u) * kRelaxedRun + (r >> 3);
 }
 
-template <int GT, int HT, bool HAS_CTL>
-__global__ __launch_bounds__(kWave) void adam_tile_relaxed_kernel(AdamArgs a, uint64_t tile0, uint32_t on_lines)
+template <int GT, int HT, bool HAS_CTL, int CACHED>
+__global__ __launch_bounds__(kWave) void adam_tile_relaxed_kernel(AdamArgs a, uint64_t tile0, uint32_t flags)
 {
     AdamConsts c = a.c;
     if (a.hyper) c = *a.hyper;
-    const uint64_t t0 = (tile0 + relaxed_tile_of_workgroup(blockIdx.x, gridDim.x)) * kWave;  // first unit of the tile
-    const uint64_t i = t0 + threadIdx.x;                                                      // this lane's 4-element unit
-    const bool out_of_place = a.p_out != a.p || a.m_out != a.m || a.v_out != a.v;
-    if constexpr (HAS_CTL) {
-        if (a.ctl->skip && !out_of_place) return;
-        c.grad_mult = a.ctl->grad_mult;
-    }
-    f32x4 p = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.p) + i);
-    f32x4 m = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.m) + i);
-    f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.v) + i);
-    bool skip = false;
-    if constexpr (HAS_CTL) skip = a.ctl->skip != 0;  // out of place: the old state still has to reach the outputs
-    if (!skip) {
-        f32x4 g;
-        if constexpr (GT == FT_F32) {
-            g = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.g) + i);
-        } else {
-            const u16x4_e w = __builtin_nontemporal_load(reinterpret_cast<const u16x4_e*>(a.g) + i);
-            g.x = half_to_float<GT>(w.x);
-            g.y = half_to_float<GT>(w.y);
-            g.z = half_to_float<GT>(w.z);
-            g.w = half_to_float<GT>(w.w);
-        }
-        adam_unit(p, g, m, v, c);
-    }
-    auto store_state = [&](float* out, f32x4 x, uint32_t bit) {
-        if (on_lines & bit)  // wave-uniform
+    const uint32_t tile = (flags & kRelaxedRuns) ? relaxed_tile_of_workgroup(blockIdx.x, gridDim.x) : blockIdx.x;
+    const uint64_t t0 = (tile0 + tile) * kWave;  // first unit of the tile
+    const uint64_t i = t0 + threadIdx.x;         // this lane's 4-element unit
+    auto store_state = [&](float* out, f32x4 x, uint32_t on_lines) {
+        if (flags & on_lines)  // wave-uniform
             st_stream(tile_rsrc(reinterpret_cast<f32x4*>(out) + t0, kWave * 16), threadIdx.x * 16, x);
         else
             __builtin_nontemporal_store(static_cast<f32x4_e>(x), reinterpret_cast<f32x4_e*>(out) + i);
     };
-    store_state(a.p_out, p, 1u);
-    store_state(a.m_out, m, 2u);
-    store_state(a.v_out, v, 4u);
+    if constexpr (HAS_CTL) {
+        if (a.ctl->skip) {
+            // A skipped step leaves the state as it is; where the outputs are other arrays than the
+            // inputs (a staging buffer on one side of the host link) the old state still has to
+            // arrive there. The low-precision copy is never written on a skip.
+            if (a.p_out != a.p) store_state(a.p_out, __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.p) + i), kRelaxedOnLinesP);
+            if (a.m_out != a.m) store_state(a.m_out, __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.m) + i), kRelaxedOnLinesM);
+            if (a.v_out != a.v) store_state(a.v_out, __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.v) + i), kRelaxedOnLinesV);
+            return;
+        }
+        c.grad_mult = a.ctl->grad_mult;
+    }
+    // Straight-line from here: the gradient unit and the three state units are fetched before
+    // anything waits for one of them.
+    f32x4 g;
+    if constexpr (GT == FT_F32) {
+        if constexpr (CACHED == 2) {
+            const __amdgpu_buffer_rsrc_t r =
+                tile_rsrc(const_cast<f32x4_e*>(reinterpret_cast<const f32x4_e*>(a.g)) + t0, kWave * 16);
+            g = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(threadIdx.x * 16), 0, 0));
+        } else {
+            g = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.g) + i);
+        }
+    } else {
+        u16x4_e w;
+        if constexpr (CACHED == 2) {
+            const __amdgpu_buffer_rsrc_t r =
+                tile_rsrc(const_cast<u16x4_e*>(reinterpret_cast<const u16x4_e*>(a.g)) + t0, kWave * 8);
+            w = __builtin_bit_cast(u16x4_e, __builtin_amdgcn_raw_buffer_load_b64(r, (int)(threadIdx.x * 8), 0, 0));
+        } else {
+            w = __builtin_nontemporal_load(reinterpret_cast<const u16x4_e*>(a.g) + i);
+        }
+        g.x = half_to_float<GT>(w.x);
+        g.y = half_to_float<GT>(w.y);
+        g.z = half_to_float<GT>(w.z);
+        g.w = half_to_float<GT>(w.w);
+    }
+    f32x4 p, m, v;
+    if constexpr (CACHED == 1) {
+        const uint32_t k = (flags >> kRelaxedCachedShift) & 3u;  // wave-uniform
+        const float* odd = k == 0 ? a.p : k == 1 ? a.m : a.v;
+        const float* first = k == 0 ? a.m : a.p;  // the other two, in order
+        const float* second = k == 2 ? a.m : a.v;
+        const __amdgpu_buffer_rsrc_t r =
+            tile_rsrc(const_cast<f32x4_e*>(reinterpret_cast<const f32x4_e*>(odd)) + t0, kWave * 16);
+        const f32x4 xo = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(threadIdx.x * 16), 0, 0));
+        const f32x4 x1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(first) + i);
+        const f32x4 x2 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(second) + i);
+        p = k == 0 ? xo : x1;
+        m = k == 0 ? x1 : (k == 1 ? xo : x2);
+        v = k == 2 ? xo : x2;
+    } else {
+        p = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.p) + i);
+        m = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.m) + i);
+        v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(a.v) + i);
+    }
+    adam_unit(p, g, m, v, c);
+    store_state(a.p_out, p, kRelaxedOnLinesP);
+    store_state(a.m_out, m, kRelaxedOnLinesM);
+    store_state(a.v_out, v, kRelaxedOnLinesV);
     if constexpr (HT == FT_F16 || HT == FT_BF16) {
-        if (!skip) {
-            const uint32_t lo = pack2<HT>(p.x, p.y), hi = pack2<HT>(p.z, p.w);
-            if (on_lines & 8u) {
-                u32x2 w;
-                w.x = lo;
-                w.y = hi;
-                st_stream(tile_rsrc(reinterpret_cast<u32x2*>(a.h) + t0, kWave * 8), threadIdx.x * 8, w);
-            } else {
-                u16x4_e w;
-                w.x = (uint16_t)(lo & 0xffffu);
-                w.y = (uint16_t)(lo >> 16);
-                w.z = (uint16_t)(hi & 0xffffu);
-                w.w = (uint16_t)(hi >> 16);
-                __builtin_nontemporal_store(w, reinterpret_cast<u16x4_e*>(a.h) + i);
-            }
+        const uint32_t lo = pack2<HT>(p.x, p.y), hi = pack2<HT>(p.z, p.w);
+        u32x2 w2;
+        w2.x = lo;
+        w2.y = hi;
+        if (flags & kRelaxedOnLinesH) {
+            st_stream(tile_rsrc(reinterpret_cast<u32x2*>(a.h) + t0, kWave * 8), threadIdx.x * 8, w2);
+        } else if (flags & kRelaxedCopyCached) {
+            st_keep(tile_rsrc(reinterpret_cast<u16x4_e*>(a.h) + t0, kWave * 8), threadIdx.x * 8, w2);
+        } else {
+            u16x4_e w;
+            w.x = (uint16_t)(lo & 0xffffu);
+            w.y = (uint16_t)(lo >> 16);
+            w.z = (uint16_t)(hi & 0xffffu);
+            w.w = (uint16_t)(hi >> 16);
+            __builtin_nontemporal_store(w, reinterpret_cast<u16x4_e*>(a.h) + i);
         }
     }
 }

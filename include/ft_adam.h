@@ -89,8 +89,8 @@ int ft_adam_destroy(int id);
  * alignments disagree (a 16-bit copy cut at an odd element, a state array one element off) are still
  * stepped tile by tile, through accesses that assume element alignment only; the tiles then start
  * where most of the traffic falls on whole cache lines (written bytes counted twice), see
- * ft_relaxed_tile_start. The same results, at 80-84 % of the memory bandwidth instead of 84-86 %
- * (measured with one array of a 202 M-element update one element off the others; 70-77 % with
+ * ft_relaxed_tile_start. The same results, at 82-85 % of the memory bandwidth instead of 85-86 %
+ * (measured with one array of a 202 M-element update one element off the others; 75 % with
  * every array at another offset).
  */
 int ft_adam_step(int id, uint64_t step, float lr, float beta1, float beta2, float eps,

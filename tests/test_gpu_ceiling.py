@@ -38,7 +38,9 @@ def _case(cases, start):
 
 
 @pytest.mark.parametrize("start,allowed", [
-    ("update,", 1.03),                        # measured 0.99-1.00
+    ("update, bf16", 1.03),                   # measured 0.99-1.00
+    ("update, m one element off", 1.06),      # 1.01-1.03: relaxed-alignment tiles, the odd state array read through the caches
+    ("update, g one element off", 1.05),      # 1.00-1.01: the same, the gradient
     ("accumulate (", 1.03),                   # 1.00-1.01
     ("accumulate + clear", 1.03),             # 1.00-1.01
     ("statistics, block partials only", 1.05),  # 1.01-1.03: the inf/nan marks beside the squares

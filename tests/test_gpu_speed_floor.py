@@ -62,8 +62,8 @@ def test_update_kernel(cuda, summary_line, variant):
 @pytest.mark.parametrize("odd_one", ["p", "m", "g", "h"])
 def test_update_with_one_array_one_element_off(cuda, summary_line, odd_one):
     """Arrays whose alignments disagree (the relaxed-alignment tiles): no caller of the reference makes
-    such views, so the floor is lower (80-84 % measured; 61-79 % before tiles started where most
-    arrays sit on cache lines and neighbouring tiles were sent to one die)."""
+    such views; 82-85.5 % measured (61-79 % before tiles started where most arrays sit on cache lines
+    and the odd array was read through the caches)."""
     from flextrain_amd import FlexTrainCPUAdam
     from flextrain_amd.memory import allocate_device_arrays
     arrays = dict(zip("pmvgh", allocate_device_arrays([(N + 4, torch.float32)] * 3 + [(N + 4, torch.bfloat16)] * 2, cuda)))
@@ -74,7 +74,7 @@ def test_update_with_one_array_one_element_off(cuda, summary_line, odd_one):
     p, m, v, g, h = (arrays[k][(1 if k == odd_one else 0):][:N] for k in "pmvgh")
     eng = FlexTrainCPUAdam(lr=1e-4)
     ms = _fastest_ms(lambda: eng._step({"step": 100}, h, p, g, m, v))
-    _check(summary_line, f"update, {odd_one} one element off the others (relaxed tiles)", ms, 28, floor=0.74)
+    _check(summary_line, f"update, {odd_one} one element off the others (relaxed tiles)", ms, 28, floor=0.78)
 
 
 def test_update_of_sixteen_contexts_in_one_launch(cuda, summary_line):

@@ -105,13 +105,29 @@ def test_many_segment_kernel_keeps_its_table_in_scalar_registers(kernels):
 
 
 def test_relaxed_alignment_kernel_uses_full_width_accesses(kernels):
-    """Arrays whose alignments disagree are still moved 16 (8) bytes per lane and instruction."""
+    """Arrays whose alignments disagree are still moved 16 (8) bytes per lane and instruction, and the
+    loads of a tile are issued back to back: the three variants differ in which array is read with the
+    default cache policy (a buffer load) instead of streaming, and must not make a load wait for the
+    one before it (a run-time choice of the load instruction per array once did: every load was
+    followed by s_waitcnt vmcnt(0))."""
     seen = 0
     for name, body in kernels.items():
         if "adam_tile_relaxed_kernel" not in name:
             continue
         seen += 1
-        assert len(re.findall(r"global_load_dwordx4 .* nt", body)) >= 3, name
+        has_ctl, cached = re.search(r"ELb([01])ELi(\d)EEEv", name).groups()  # the last two template arguments
+        has_ctl, cached = has_ctl == "1", int(cached)
+        fp32_g = "kernelILi0E" in name
+        streaming = len(re.findall(r"global_load_dwordx4 .* nt", body))
+        buffered = len(re.findall(r"buffer_load_dwordx[24] ", body))
+        # a skipped out-of-place step copies the three state arrays through: three more streaming loads
+        assert streaming == 3 + (1 if fp32_g else 0) - (1 if cached == 1 else 0) - (1 if cached == 2 and fp32_g else 0) \
+            + (3 if has_ctl else 0), name
+        assert buffered == (1 if cached else 0), name
         assert len(re.findall(r"global_store_dwordx4 .* nt", body)) >= 3, name
         assert not re.search(r"global_(load|store)_(ubyte|short|ushort)", body), name
-    assert seen == 3 * 3 * 2
+        assert "flat_load" not in body and "flat_store" not in body, name
+        # the four loads of a tile (gradient, p, m, v) follow one another with no wait for a load between them
+        loads = [m.start() for m in re.finditer(r"(global|buffer)_load_dwordx[24] ", body)]
+        assert any("s_waitcnt vmcnt" not in body[loads[k]:loads[k + 3]] for k in range(len(loads) - 3)), name
+    assert seen == 3 * 3 * 2 * 3
