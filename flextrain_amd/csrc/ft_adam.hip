@@ -82,6 +82,23 @@ constexpr int kMaxStatsBlocks = 8192;
 
 inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 inline size_t elem_size(int dt) { return dt == FT_F32 ? 4 : 2; }
+
+// True when, `head` elements in, every array of a step sits on a cache line (the 16-bit copy, which
+// is only written: on half a line), or when the segment is too short for that to matter. Vector
+// alignment is not all: the aligned kernels stream every array, and an array whose tiles start
+// inside a line (m sixteen bytes off p, say) then costs them far more than it costs the relaxed
+// kernel, which knows how to treat such an array (measured on 202 M elements with one array 4
+// elements off the others: m 0.895 ms, p 1.04 ms, against 0.838 and 0.844 ms; the aligned kernel is at
+// full speed with the copy 64 bytes off, 0.828 ms, and not with a state array 64 bytes off, 0.857 ms).
+inline bool arrays_on_lines(size_t head, size_t n, const void* p, const void* m, const void* v, const void* g, size_t gsz,
+                            const void* h, const void* out_p, const void* out_m, const void* out_v)
+{
+    if (head >= n || n - head < 16 * 256) return true;
+    auto on = [&](const void* base, size_t esz, size_t line) { return aligned(static_cast<const char*>(base) + head * esz, line); };
+    const size_t line = fth::kLineBytes;
+    return on(p, 4, line) && on(m, 4, line) && on(v, 4, line) && on(g, gsz, line) && (h == nullptr || on(h, 2, line / 2)) &&
+           on(out_p, 4, line) && on(out_m, 4, line) && on(out_v, 4, line);
+}
 inline bool valid_dtype(int dt) { return dt == FT_F32 || dt == FT_F16 || dt == FT_BF16; }
 
 }  // namespace
@@ -245,7 +262,9 @@ int launch_typed(const ftk::AdamConsts& c, float* p, const void* g, float* m, fl
         return FT_OK;
     };
 
-    if (!vec_ok) {
+    // Segments whose arrays agree as vectors but not on cache lines go the relaxed way as well.
+    const bool lines_ok = arrays_on_lines(head, n, p, m, v, g, gsz, h, out.p, out.m, out.v);
+    if (!vec_ok || !lines_ok) {
         // Arrays whose alignments disagree: whole tiles still go through a tile kernel (one that
         // assumes element alignment only), the rest element by element. The tiles start where most
         // of the traffic is on whole cache lines (written bytes counted twice).
@@ -817,9 +836,9 @@ int ft_adam_step_multi(int id, const ft_adam_segment_t* segs, int n_segs, int g_
                             (!hb || aligned(hb + head * 2, 8));
         const size_t body_tiles = (sg.n - head) / (ftk::kWave * 4);
         const bool edge = head + (sg.n - head) % (ftk::kWave * 4) > 0;
-        if (!vec_ok || body_tiles + 1 > multi_launch_limit()) {
-            // arrays whose alignments disagree, or a segment too long for one grid: the
-            // single-segment path takes it
+        if (!vec_ok || !arrays_on_lines(head, sg.n, p, mb, vb, gb, gsz, hb, p, mb, vb) || body_tiles + 1 > multi_launch_limit()) {
+            // arrays whose alignments disagree (as vectors or on cache lines), or a segment too long
+            // for one grid: the single-segment path takes it
             rc = fth::launch_adam(c, p, sg.g, g_dtype, static_cast<float*>(sg.m), static_cast<float*>(sg.v), sg.half_out,
                                   half_dtype, sg.n, ctl, stream, nullptr, nullptr, nullptr,
                                   static_cast<const ftk::AdamConsts*>(sg.hyper));

@@ -143,12 +143,13 @@ def test_mismatched_alignment_keeps_the_results(cuda, oracle):
     for odd in "pgmvh" if not (odd == "h" and h is None)])
 @pytest.mark.parametrize("control", [None, "scale", "skip"])
 def test_one_array_off_the_others(cuda, oracle, odd_one, g_dtype, half_dtype, control):
-    """One array starts 1, 2 or 3 elements into its buffer, the others at the start of theirs (a
-    16-bit copy cut at an odd element, a state array one element off): many tiles, bits as the
+    """One array starts 1, 2, 3, 4 or 16 elements into its buffer, the others at the start of theirs (a
+    16-bit copy cut at an odd element, a state array one element off; with 4 and 16 the arrays agree
+    as vectors and disagree on cache lines, which takes the same kernel): many tiles, bits as the
     oracle's, nothing written outside the views, a skipped step leaves everything alone."""
     eng = _engine(**HP)
-    n, pad = 300_003, 8
-    for shift in (1, 2, 3):
+    n, pad = 300_003, 24
+    for shift in (1, 2, 3, 4, 16):
         P, G, M, V = _gen(n + pad, cuda, seed=40 + shift, g_dtype=g_dtype)
         H = torch.full((n + pad,), 7.0, dtype=half_dtype, device=cuda) if half_dtype is not None else None
         offs = {k: (shift if k == odd_one else 0) for k in "pgmvh"}
