@@ -1031,6 +1031,9 @@ int grad_accumulate_impl(void* acc, int acc_dtype, void* g, int g_dtype, size_t 
         if (n - head >= 16 * 256) {
             const size_t tile_bytes = 256 * asz;
             head = ((tile_bytes - (reinterpret_cast<uintptr_t>(acc) & (tile_bytes - 1))) & (tile_bytes - 1)) / asz;
+            // ... and g aligned as vectors but off the cache lines there is treated like g off its
+            // vector alignment: its tiles share lines with their neighbours all the same
+            if (!aligned(static_cast<char*>(g) + head * gsz, fth::kLineBytes)) g_relaxed = true;
         }
         nvec = (n - head) / 4;
     }

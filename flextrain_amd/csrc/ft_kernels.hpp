@@ -980,21 +980,28 @@ __device__ __forceinline__ void accumulate_tile(void* acc, void* g, uint64_t til
     const uint64_t i = t0 + threadIdx.x;
     if (threadIdx.x >= live) return;
 
-    // The gradient unit as raw bits, fetched either way before anything waits for it (g_relaxed: g
-    // does not reach its vector alignment where acc does, so element alignment only).
-    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    // The gradient unit as raw bits, fetched either way before anything waits for it. g_relaxed: g's
+    // tiles do not start on cache lines where acc's do (g off its vector alignment, or only off the
+    // lines), so element alignment only, and a tile shares a line with its neighbour at either end:
+    // read with the default cache policy (a buffer load: a distinct instruction, the compiler would
+    // merge two global loads that differ in the streaming hint), so that the second reader finds the
+    // line in a cache and the clearing store below meets it there.
     f32x4 g32;
     u32x2 g16;
     if constexpr (GT == FT_F32) {
-        if (!g_relaxed)
+        if (!g_relaxed) {
             g32 = ld<true>(reinterpret_cast<const f32x4*>(g) + i);
-        else
-            g32 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_e*>(g) + i);
+        } else {
+            const __amdgpu_buffer_rsrc_t r = tile_rsrc(reinterpret_cast<f32x4_e*>(g) + t0, live * 16);
+            g32 = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(threadIdx.x * 16), 0, 0));
+        }
     } else {
-        if (!g_relaxed)
+        if (!g_relaxed) {
             g16 = ld<true>(reinterpret_cast<const u32x2*>(g) + i);
-        else
-            g16 = __builtin_bit_cast(u32x2, static_cast<u16x4>(__builtin_nontemporal_load(reinterpret_cast<const u16x4_e*>(g) + i)));
+        } else {
+            const __amdgpu_buffer_rsrc_t r = tile_rsrc(reinterpret_cast<u16x4_e*>(g) + t0, live * 8);
+            g16 = __builtin_amdgcn_raw_buffer_load_b64(r, (int)(threadIdx.x * 8), 0, 0);
+        }
     }
     f32x4 a4;
     if constexpr (AT == FT_F32) {

@@ -177,9 +177,10 @@ int ft_release_stream_scratch(void* stream);
  * receive buffer (coordinator/optimizer.py:743). With stats_out != NULL the pass also produces the
  * statistics ft_grad_stats would report for the new acc (pre-multiplied by stats_pre_mult), so
  * the last accumulation of a step makes the separate statistics pass unnecessary.
- * acc and g should start at the same element offset modulo 4 of their buffers (then both are moved
- * with aligned vector accesses); a g that does not is read and cleared through accesses that assume
- * element alignment only, with the same results. With statistics the
+ * acc and g should start at the same element offset of their buffers (then both are moved with
+ * aligned vector accesses and every tile covers whole cache lines of both); a g that does not is
+ * read (through the caches rather than streamed) and cleared through accesses that assume element
+ * alignment only, with the same results, 1-3 % slower. With statistics the
  * workspace must hold ft_grad_accumulate_workspace_bytes(n) bytes (16 bytes per 256 elements on
  * top of the fixed part), or be NULL for the library's own buffer. */
 size_t ft_grad_accumulate_workspace_bytes(size_t n);
