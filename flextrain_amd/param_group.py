@@ -310,3 +310,6 @@ class StepContextContainer(Sequence):
 
     def __len__(self) -> int:
         return len(self._grouped_step_contexts)
+
+    def __iter__(self):
+        return iter(self._grouped_step_contexts)
