@@ -207,6 +207,8 @@ def test_step_context_container_partitions_evenly(arg, parts):
             got += len(idx)
         assert got == share
     assert (seen == 1).all()
+    # iterating the container goes over its parts and ends (indexing asserts its range, as the reference's does)
+    assert [id(part) for part in container] == [id(container[k]) for k in range(parts)]
     # re-planning with half_parameter=None yields contexts without a copy-out
     container.plan(None, full, grad, states)
     assert all(ctx.half_parameter is None for k in range(parts) for ctx in container[k])
