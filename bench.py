@@ -812,8 +812,9 @@ def bench_resident7b(args, torch, dev) -> int:
 def measure_resident(torch, dev, workload, steps, warmup, calibration_copy=False):
     """cfg2 / cfg3 / cfg4 with everything resident in HBM: `warmup` untimed steps, then `steps` timed
     ones with HIP events on the stream the kernels run on (torch's current stream), recorded inside
-    the timed region: one in front of the statistics pass (when the workload has one), one in front
-    of the update, one behind it."""
+    the timed region: one in front of every step and one behind it. A workload with a statistics pass
+    then runs the same steps once more with a third event between the pass and the update, for the
+    two parts, and the pass `steps` times by itself."""
     from flextrain_amd import FlexTrainCPUAdam
     from flextrain_amd.loss_scaler import GradientGuard
     eng = FlexTrainCPUAdam(**HP)
@@ -854,27 +855,34 @@ def measure_resident(torch, dev, workload, steps, warmup, calibration_copy=False
         one_step()
     torch.cuda.synchronize()
 
+    # The timed region: `steps` steps, one event in front of each and one behind it.
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
           for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        if guard is not None:
+        ev[i][0].record()
+        one_step()
+        ev[i][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    whole_ms = [e[0].elapsed_time(e[2]) for e in ev]
+    if guard is not None:
+        # The two parts of a guarded step, from a second run of the same steps with a third event
+        # between the statistics pass and the update (an event between two kernels is a bubble of its
+        # own, about 10 us: it stays out of the timed region above).
+        for i in range(steps):
             ev[i][0].record()
             guard.begin()
             ctl = guard.add_and_decide(g, loss_scale=scale, max_grad_norm=max_norm)
             ev[i][1].record()
             eng._step(group, h, p, g, m, v, control=ctl)
-        else:  # no statistics pass: one event pair around the update is all there is to time
-            ev[i][1].record()
-            eng._step(group, h, p, g, m, v)
-        ev[i][2].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    upd_ms = [e[1].elapsed_time(e[2]) for e in ev]
-    pre_ms = [e[0].elapsed_time(e[1]) for e in ev] if guard is not None else [0.0]
-    whole_ms = [e[0].elapsed_time(e[2]) for e in ev] if guard is not None else upd_ms
+            ev[i][2].record()
+        torch.cuda.synchronize()
+        upd_ms = [e[1].elapsed_time(e[2]) for e in ev]
+        pre_ms = [e[0].elapsed_time(e[1]) for e in ev]
+    else:
+        upd_ms, pre_ms = whole_ms, [0.0]
     # The statistics pass by itself: `steps` launches back to back between ONE pair of events. (Inside
     # a step the event between the two kernels and the update that has just finished writing 2.8 GB
     # cost the short pass 5-10 us that are not the kernel's.)
@@ -899,8 +907,10 @@ def measure_resident(torch, dev, workload, steps, warmup, calibration_copy=False
 
 def guarded_step_record(r):
     """Compact record of a step with a statistics pass in front (cfg3, cfg4): the whole step between
-    the first and the last HIP event, its two parts, and the fraction of the HBM peak at the step's
-    30 algorithmic bytes per element (2 for the statistics read, 28 for the update)."""
+    one HIP event in front of it and one behind it, its two parts (from a second run with an event
+    between them, which costs a bubble of its own: the parts add up to more than the step), and the
+    fraction of the HBM peak at the step's 30 algorithmic bytes per element (2 for the statistics
+    read, 28 for the update)."""
     n = r["n"]
     whole = r["whole_avg"]
     return {"workload": r["name"], "elements": n, "steps": r["steps"], "warmup": r["warmup"],
