@@ -624,8 +624,9 @@ __device__ __forceinline__ void stats_accumulate_finite(u32x4 w, float pre_mult,
     }
 }
 
-// Block-level end of a statistics pass: per-lane fp64 sums and counts -> the block's totals, added
-// in a fixed tree order through LDS; valid in thread 0.
+// Block-level end of a statistics pass: per-lane fp64 sums and counts -> the block's totals: a
+// wavefront sum each (DPP, fixed order), then the wavefronts' sums in order through LDS; valid in
+// thread 0.
 template <int BLOCK>
 __device__ __forceinline__ void block_stats_reduce(double lane_sum, uint32_t bad, double& total, uint64_t& total_bad)
 {
@@ -796,7 +797,7 @@ struct StatsFinalArgs {
 };
 
 // End of a statistics pass, run by the first 256 threads of ONE block (all threads of the block must
-// call it): adds the block partials in a fixed tree order, then the elements before/after the vector
+// call it): adds the block partials in a fixed order (strided per thread, wavefront sums, then the four wavefronts), then the elements before/after the vector
 // body one by one, and writes or accumulates the result. The order of the additions depends on
 // nparts only, not on which block runs it.
 template <int GT, bool COHERENT>
