@@ -797,9 +797,10 @@ struct StatsFinalArgs {
 };
 
 // End of a statistics pass, run by the first 256 threads of ONE block (all threads of the block must
-// call it): adds the block partials in a fixed order (strided per thread, wavefront sums, then the four wavefronts), then the elements before/after the vector
-// body one by one, and writes or accumulates the result. The order of the additions depends on
-// nparts only, not on which block runs it.
+// call it): adds the block partials in a fixed order (strided per thread, wavefront sums, then the
+// four wavefronts), then the elements before/after the vector body one by one, and writes or
+// accumulates the result. The order of the additions depends on nparts only, not on which block
+// runs it.
 template <int GT, bool COHERENT>
 __device__ __forceinline__ void stats_final_block(const StatsPartial* partials, int nparts, float pre_mult, const StatsFinalArgs& f)
 {
