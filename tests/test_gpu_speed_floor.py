@@ -74,7 +74,7 @@ def test_update_with_one_array_one_element_off(cuda, summary_line, odd_one):
     p, m, v, g, h = (arrays[k][(1 if k == odd_one else 0):][:N] for k in "pmvgh")
     eng = FlexTrainCPUAdam(lr=1e-4)
     ms = _fastest_ms(lambda: eng._step({"step": 100}, h, p, g, m, v))
-    _check(summary_line, f"update, {odd_one} one element off the others (relaxed tiles)", ms, 28, floor=0.78)
+    _check(summary_line, f"update, {odd_one} one element off the others (relaxed tiles)", ms, 28, floor=0.75)
 
 
 def test_update_of_sixteen_contexts_in_one_launch(cuda, summary_line):
