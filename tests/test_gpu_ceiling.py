@@ -38,12 +38,12 @@ def _case(cases, start):
 
 
 @pytest.mark.parametrize("start,allowed", [
-    ("update, bf16", 1.03),                   # measured 0.99-1.00
-    ("update, m one element off", 1.06),      # 1.01-1.03: relaxed-alignment tiles, the odd state array read through the caches
-    ("update, g one element off", 1.05),      # 1.00-1.01: the same, the gradient
-    ("accumulate (", 1.03),                   # 1.00-1.01
-    ("accumulate + clear", 1.03),             # 1.00-1.01
-    ("statistics, block partials only", 1.05),  # 1.01-1.03: the inf/nan marks beside the squares
+    ("update, bf16", 1.04),                   # measured 0.99-1.00
+    ("update, m one element off", 1.07),      # 1.01-1.02: relaxed-alignment tiles, the odd state array read through the caches
+    ("update, g one element off", 1.05),      # 0.99-1.00: the same, the gradient
+    ("accumulate (", 1.05),                   # 1.01-1.015
+    ("accumulate + clear", 1.05),             # 1.01
+    ("statistics, block partials only", 1.06),  # 1.00-1.03: the inf/nan marks beside the squares
 ])
 def test_kernel_keeps_up_with_its_bare_twin(cases, summary_line, start, allowed):
     rec = _case(cases, start)
@@ -59,4 +59,4 @@ def test_statistics_pass_pays_a_few_microseconds_for_its_final_sum(cases, summar
     rec = _case(cases, "statistics with final sum")
     extra = rec["shipped_us"] - rec["bare_us"]
     summary_line(f"ceiling, {rec['case']}: shipped {rec['shipped_us']:.1f} us, bare {rec['bare_us']:.1f} us (+{extra:.1f} us)")
-    assert extra <= 7.0, rec
+    assert extra <= 8.0, rec
