@@ -177,6 +177,29 @@ def test_one_array_off_the_others(cuda, oracle, odd_one, g_dtype, half_dtype, co
         assert torch.equal(G, before["g"])
 
 
+@pytest.mark.parametrize("odd_one", ["m", "g", "h", "pv"])
+def test_relaxed_tiles_over_several_steps(cuda, oracle, odd_one):
+    """The relaxed-alignment tiles read the array that is off the cache lines through the caches, and
+    neighbouring tiles on different dies share a line of it: five steps in a row on the same arrays
+    (each reading what the one before wrote, other arrays updated in between) stay bit for bit with
+    the oracle."""
+    eng = _engine(**HP)
+    n, pad = 1_000_003, 8
+    P, G, M, V = _gen(n + pad, cuda, seed=77, g_dtype=torch.bfloat16)
+    H = torch.zeros(n + pad, dtype=torch.bfloat16, device=cuda)
+    offs = {k: (1 if k in odd_one else 0) for k in "pgmvh"}
+    p, g, m, v, h = (t[offs[k]:offs[k] + n] for k, t in (("p", P), ("g", G), ("m", M), ("v", V), ("h", H)))
+    pn, mn, vn = to_np(p).copy(), to_np(m).copy(), to_np(v).copy()
+    hn = np.zeros(n, np.uint16)
+    for step in range(1, 6):
+        g.copy_((torch.randn(n, device=cuda, generator=torch.Generator(device=cuda).manual_seed(step)) * 1e-3).to(torch.bfloat16))
+        oracle.adam_step(pn, to_np(g), mn, vn, step=step, lr=HP["lr"], betas=HP["betas"], eps=HP["eps"],
+                         weight_decay=HP["weight_decay"], bias_correction=HP["bias_correction"], adamw_mode=True,
+                         g_dtype=CODE[torch.bfloat16], half_out=hn, half_dtype=CODE[torch.bfloat16])
+        eng._step({"step": step}, h, p, g, m, v)
+    _compare(f"{odd_one} off, five steps", (p, m, v, h), (pn, mn, vn, hn), torch.bfloat16)
+
+
 def test_special_values(cuda, oracle):
     """Zeros, denormals, huge and tiny magnitudes, negative zero; g = m = v = 0 leaves m = v = 0 and
     p' = fma(p, -lr*wd, p) exactly (what happens to the zero padding at the end of a unit)."""
