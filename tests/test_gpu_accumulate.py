@@ -97,6 +97,32 @@ def test_gradients_off_the_accumulators_alignment(cuda, oracle, acc_dtype, g_dty
         guard.accumulate(torch.zeros(1000, device=cuda), torch.zeros(1001, device=cuda, dtype=torch.bfloat16))  # lengths differ
 
 
+@pytest.mark.parametrize("g_off", [1, 4, 32])
+def test_micro_batches_into_an_accumulator_the_gradients_are_off(cuda, oracle, g_off):
+    """Four micro-batches in a row, the gradient buffer off the accumulator's cache lines (by one
+    element, by 8 bytes, by 64): it is read through the caches and cleared by every pass, refilled by
+    another kernel in between; the accumulator stays bit for bit with the oracle and the buffer ends
+    cleared."""
+    from flextrain_amd.loss_scaler import GradientGuard
+    guard = GradientGuard(cuda)
+    n = 1_000_003
+    A = torch.zeros(n + 64, device=cuda)
+    G = torch.zeros(n + 64, device=cuda, dtype=torch.bfloat16)
+    a, g = A[:n], G[g_off:g_off + n]
+    an = np.zeros(n, np.float32)
+    for mb in range(4):
+        g.copy_((torch.randn(n, device=cuda, generator=torch.Generator(device=cuda).manual_seed(100 + mb)) * 0.1).to(torch.bfloat16))
+        gn = _bits(g).copy()
+        oracle.grad_accumulate(an, CODE[torch.float32], gn, CODE[torch.bfloat16], scale=0.25, zero_g=True)
+        guard.begin()
+        guard.accumulate(a, g, scale=0.25, zero_grads=True, with_stats=mb == 3)
+        assert max_ulp_gpu(a, an) == 0, mb
+        assert not bool(G.view(torch.int16).any()), mb
+    d = guard.decide()
+    bad, sumsq = oracle.grad_stats(an, CODE[torch.float32])
+    assert d.nonfinite == bad == 0 and abs(d.sumsq - sumsq) <= 2 * NORM_RTOL * sumsq
+
+
 def test_accumulate_llama7b_layer(cuda, oracle):
     """Full-size: fp32 accumulator += bf16 gradients over the 7B-layer partition, with the
     statistics of the result gathered in the same pass."""
