@@ -19,7 +19,7 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 def test_help_names_every_workload():
     res = _run("--help")
     assert res.returncode == 0
-    for name in ("cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate", "resident7b", "--steps", "--warmup", "--gpus"):
+    for name in ("cfg2", "cfg3", "cfg4", "cfg5", "pipeline", "accumulate", "resident7b", "multi", "ceilings", "--steps", "--warmup", "--gpus"):
         assert name in res.stdout
 
 
